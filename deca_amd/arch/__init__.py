@@ -1,0 +1,4 @@
+from .Arch import Arch
+from .MI355X import MI355X
+
+__all__ = ["Arch", "MI355X"]

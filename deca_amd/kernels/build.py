@@ -1,0 +1,167 @@
+"""
+Shared compilation helpers for the hand-written HIP kernel templates.
+
+Counterpart of the reference's src/kernels/build.py (nvcc callback :56-64,
+`build_kernel` :73-87, `cuda_target` :67-70): a kernel is a `.hip` template
+under `deca_amd/csrc/` specialised with `-D` macros and compiled by
+`hipcc --genco` into a gfx950 code object.  Nothing here imports torch or
+touches the GPU, so it is safe inside spawned compile workers.
+"""
+
+from __future__ import annotations
+
+import hashlib
+import os
+import shutil
+import subprocess
+import tempfile
+from dataclasses import dataclass, field
+
+PKG_ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CSRC_DIR = os.path.join(PKG_ROOT, "csrc")
+CACHE_DIR = os.path.join(PKG_ROOT, "_kcache")
+KERNEL_SYMBOL = "deca_main"
+DEFAULT_ARCH = "gfx950"
+
+# The reference passes --use_fast_math to nvcc (build.py:9).
+FAST_MATH_OPTIONS = ["-ffast-math"]
+# Packed-FP32 VALU forms are switched off for every device compile.
+BASE_OPTIONS = ["-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+@dataclass(frozen=True)
+class KernelSpec:
+    """Everything needed to compile and launch one specialised kernel.
+
+    Plays the role of the IRModule returned by the reference's `make_*`
+    functions: the template plus its compile-time constants, and the launch
+    geometry the reference derives in gemm_tir.py:156, rowwise_tir.py:128 and
+    flash_attn_tir.py:147.
+    """
+
+    template: str  # file name under csrc/
+    defines: tuple  # ((name, value), ...) sorted
+    grid: tuple  # (gx, gy, gz)
+    block: tuple  # (bx, by, bz)
+    nargs: int  # device pointers the kernel takes
+    lds_bytes: int = 0  # dynamic LDS (static LDS lives in the code object)
+    options: tuple = tuple(FAST_MATH_OPTIONS)
+    symbol: str = KERNEL_SYMBOL
+    meta: tuple = field(default=(), compare=False)  # free-form (name, value) notes
+
+    @property
+    def source_path(self) -> str:
+        return os.path.join(CSRC_DIR, self.template)
+
+    def define_flags(self) -> list[str]:
+        return [f"-D{k}={v}" for k, v in self.defines]
+
+    def key(self) -> str:
+        """Content hash: template text + macros + options."""
+        h = hashlib.sha1()
+        with open(self.source_path, "rb") as f:
+            h.update(f.read())
+        h.update(repr((self.defines, self.options, BASE_OPTIONS)).encode())
+        return h.hexdigest()[:20]
+
+    def show(self) -> str:
+        defs = " ".join(self.define_flags())
+        return f"{self.template} grid={self.grid} block={self.block} lds={self.lds_bytes}\n  {defs}"
+
+
+def make_spec(template, defines: dict, grid, block, nargs, lds_bytes=0, options=None, meta=None):
+    def norm(v):
+        if isinstance(v, bool):
+            return int(v)
+        return v
+
+    return KernelSpec(
+        template=template,
+        defines=tuple(sorted((k, norm(v)) for k, v in defines.items())),
+        grid=tuple(int(g) for g in grid),
+        block=tuple(int(b) for b in block),
+        nargs=int(nargs),
+        lds_bytes=int(lds_bytes),
+        options=tuple(FAST_MATH_OPTIONS if options is None else options),
+        meta=tuple(sorted((meta or {}).items())),
+    )
+
+
+def rocm_target(device_id: int = 0) -> str:
+    """Offload architecture of the visible device (reference: `cuda_target`, build.py:67-70)."""
+    from deca_amd.driver.driver import get_driver
+
+    arch = get_driver().device_info(device_id).gcn_arch
+    return arch.split(":")[0] or DEFAULT_ARCH
+
+
+def hipcc_path() -> str:
+    for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and os.path.exists(cand):
+            return cand
+    raise RuntimeError("hipcc not found (set HIPCC or add /opt/rocm/bin to PATH)")
+
+
+def compile_command(spec: KernelSpec, arch: str, out_path: str) -> list[str]:
+    return [
+        hipcc_path(), "--genco", f"--offload-arch={arch}", *BASE_OPTIONS, *spec.options,
+        *spec.define_flags(), spec.source_path, "-o", out_path,
+    ]
+
+
+def build_kernel(spec: KernelSpec, arch: str | None, path: str, dump_dir: str | None = None) -> str:
+    """Compiles `spec` into the code object `path`; `dump_dir` keeps the
+    generated ISA (`*.s`) for inspection (reference: build.py:73-87)."""
+    arch = arch or DEFAULT_ARCH
+    os.makedirs(os.path.dirname(os.path.abspath(path)) or ".", exist_ok=True)
+    tmp = f"{path}.tmp{os.getpid()}"
+    cmd = compile_command(spec, arch, tmp)
+    cwd = None
+    if dump_dir:
+        os.makedirs(dump_dir, exist_ok=True)
+        cmd.append("--save-temps")
+        cwd = dump_dir
+    proc = subprocess.run(cmd, capture_output=True, text=True, cwd=cwd)
+    if proc.returncode != 0:
+        if os.path.exists(tmp):
+            os.remove(tmp)
+        raise RuntimeError(f"hipcc failed for {spec.show()}:\n{proc.stderr[-4000:]}")
+    os.replace(tmp, path)
+    return path
+
+
+def cached_build(spec: KernelSpec, arch: str | None = None) -> str:
+    """Path of the code object of `spec` in the in-tree cache, compiling on a miss."""
+    arch = arch or DEFAULT_ARCH
+    path = os.path.join(CACHE_DIR, f"{os.path.splitext(spec.template)[0]}_{arch}_{spec.key()}.hsaco")
+    if not os.path.exists(path):
+        build_kernel(spec, arch, path)
+    return path
+
+
+def kernel_resources(spec: KernelSpec, arch: str | None = None) -> dict:
+    """Compiles `spec` to assembly and returns the resource usage the code
+    object records (VGPRs, AGPRs, SGPRs, LDS, spills).  Host only."""
+    arch = arch or DEFAULT_ARCH
+    with tempfile.TemporaryDirectory(prefix="deca_res_") as d:
+        asm = os.path.join(d, "k.s")
+        cmd = [
+            hipcc_path(), "-S", "--cuda-device-only", f"--offload-arch={arch}", *BASE_OPTIONS,
+            *spec.options, *spec.define_flags(), spec.source_path, "-o", asm,
+        ]
+        proc = subprocess.run(cmd, capture_output=True, text=True)
+        if proc.returncode != 0:
+            raise RuntimeError(f"hipcc failed for {spec.show()}:\n{proc.stderr[-4000:]}")
+        out = {}
+        keys = {
+            ".vgpr_count:": "vgprs", ".agpr_count:": "agprs", ".sgpr_count:": "sgprs",
+            ".group_segment_fixed_size:": "lds_bytes", ".private_segment_fixed_size:": "scratch_bytes",
+            ".vgpr_spill_count:": "vgpr_spills", ".sgpr_spill_count:": "sgpr_spills",
+        }
+        with open(asm) as f:
+            for line in f:
+                s = line.strip()
+                for k, name in keys.items():
+                    if s.startswith(k):
+                        out[name] = int(s.split()[-1])
+        return out

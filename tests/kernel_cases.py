@@ -1,0 +1,55 @@
+"""Kernel specialisations the GPU tests use, listed in one place so that the
+build step can compile all of them ahead of the GPU run."""
+
+from deca_amd.kernels.rowwise_hip import RowConfig, make_rowwise
+
+# (op, M, N, dtype, cfg)
+ROWWISE_CASES = [
+    # reg mode, the benchmark row lengths at a CPU-checkable row count
+    ("softmax", 256, 4096, "float16", RowConfig(128, 1, 8)),
+    ("softmax", 256, 4096, "float16", RowConfig(64, 1, 8)),
+    ("softmax", 256, 4096, "float16", RowConfig(256, 2, 8)),
+    ("softmax", 256, 4096, "float16", RowConfig(512, 2, 8, hint=True)),
+    ("softmax", 256, 4096, "bfloat16", RowConfig(128, 2, 8)),
+    ("softmax", 256, 4096, "float16", RowConfig(128, 4, 4)),
+    ("softmax", 256, 4096, "float16", RowConfig(1024, 1, 4)),
+    # rows owned by a slice of a wave
+    ("softmax", 512, 256, "float16", RowConfig(16, 8, 8)),
+    ("softmax", 512, 1024, "float16", RowConfig(32, 4, 8)),
+    # ragged rows: the last chunk is out of the row for the upper lanes
+    ("softmax", 128, 1000, "float16", RowConfig(64, 2, 8)),
+    ("softmax", 128, 4104, "bfloat16", RowConfig(128, 1, 8)),
+    ("softmax", 64, 32000, "float16", RowConfig(256, 1, 8, "twopass", 4)),
+    ("softmax", 64, 32000, "float16", RowConfig(1024, 1, 8, "twopass", 2, True)),
+    ("softmax", 64, 32000, "float16", RowConfig(1024, 1, 8, "reg")),
+    ("softmax", 16, 128256, "bfloat16", RowConfig(1024, 1, 8, "twopass", 4)),
+    ("softmax", 256, 4096, "float16", RowConfig(64, 4, 8, "twopass", 2)),
+    ("softmax", 256, 4096, "float16", RowConfig(128, 1, 4, "twopass", 1, True)),
+    # single-row and single-block extremes
+    ("softmax", 4, 128, "float16", RowConfig(16, 4, 8)),
+    ("rmsnorm", 256, 4096, "bfloat16", RowConfig(128, 1, 8)),
+    ("rmsnorm", 256, 4096, "bfloat16", RowConfig(64, 2, 8, hint=True)),
+    ("rmsnorm", 256, 4096, "float16", RowConfig(256, 1, 8)),
+    ("rmsnorm", 256, 8192, "float16", RowConfig(512, 1, 8)),
+    ("rmsnorm", 256, 8192, "float16", RowConfig(1024, 1, 8)),
+    ("rmsnorm", 256, 8192, "float16", RowConfig(128, 2, 4)),
+    ("rmsnorm", 128, 1000, "bfloat16", RowConfig(64, 2, 8)),
+    ("rmsnorm", 512, 1024, "float16", RowConfig(32, 2, 8)),
+    ("rmsnorm", 256, 4096, "bfloat16", RowConfig(64, 4, 8, "twopass", 2)),
+    ("rmsnorm", 64, 32000, "float16", RowConfig(512, 2, 8, "twopass", 4, True)),
+]
+
+# Full-size benchmark shapes (property checks + a sampled comparison).
+ROWWISE_FULL = [
+    ("softmax", 16384, 4096, "float16", RowConfig(128, 1, 8)),
+    ("rmsnorm", 16384, 4096, "bfloat16", RowConfig(128, 1, 8)),
+    ("rmsnorm", 8192, 8192, "float16", RowConfig(256, 1, 8)),
+]
+
+
+def rowwise_specs(eps: float = 1e-6):
+    return [make_rowwise(op, M, N, dt, cfg, eps) for op, M, N, dt, cfg in ROWWISE_CASES + ROWWISE_FULL]
+
+
+def all_specs():
+    return rowwise_specs()
