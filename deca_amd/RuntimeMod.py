@@ -37,9 +37,7 @@ class RuntimeMod:
 
     @property
     def is_flash_attn(self) -> bool:
-        from deca_amd.operators.FlashAttention import FlashAttention
-
-        return isinstance(self.operator, FlashAttention)
+        return bool(getattr(self.operator, "is_attention", False))
 
     @property
     def is_kernel_op(self) -> bool:

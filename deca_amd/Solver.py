@@ -1,0 +1,243 @@
+"""
+Enumerates the valid kernel configurations of one operator at one shape.
+
+Same entry points as the reference's src/Solver.py (`solve_rowwise` :389,
+`solve_gemm_tc` :473, `solve_flash_attn` :304), with the constraint sets
+re-derived for CDNA4: 64-lane waves, a 512-entry unified VGPR file per lane and
+SIMD shared by the resident waves, 160 KiB of LDS per CU with no L1 carve-out.
+
+Each constraint set is written once against a tiny expression interface
+(`_IntOps` on Python ints, `_Z3Ops` on Z3 bit-vectors).  When z3 is importable
+the all-SAT loop with blocking clauses of the reference is used; otherwise the
+(small, finite) domain product is enumerated exhaustively.  Both return the
+same set; results are sorted so that the order does not depend on the solver.
+Importing this module touches no GPU.
+"""
+
+from __future__ import annotations
+
+import itertools
+
+try:  # pragma: no cover - z3 is optional
+    import z3 as _z3
+except Exception:  # noqa: BLE001
+    _z3 = None
+
+
+# ---------------------------------------------------------------------------
+# expression interface
+# ---------------------------------------------------------------------------
+class _IntOps:
+    @staticmethod
+    def const(v):
+        return int(v)
+
+    @staticmethod
+    def udiv(a, b):
+        return a // b
+
+    @staticmethod
+    def urem(a, b):
+        return a % b
+
+    @staticmethod
+    def ule(a, b):
+        return a <= b
+
+    @staticmethod
+    def uge(a, b):
+        return a >= b
+
+    @staticmethod
+    def eq(a, b):
+        return a == b
+
+    @staticmethod
+    def ite(c, a, b):
+        return a if c else b
+
+    @staticmethod
+    def implies(a, b):
+        return (not a) or b
+
+    @staticmethod
+    def all_of(*xs):
+        return all(xs)
+
+    @staticmethod
+    def any_of(*xs):
+        return any(xs)
+
+
+class _Z3Ops:  # pragma: no cover - exercised only when z3 is installed
+    BITS = 32
+
+    @classmethod
+    def const(cls, v):
+        return _z3.BitVecVal(int(v), cls.BITS)
+
+    @staticmethod
+    def udiv(a, b):
+        return _z3.UDiv(a, b)
+
+    @staticmethod
+    def urem(a, b):
+        return _z3.URem(a, b)
+
+    @staticmethod
+    def ule(a, b):
+        return _z3.ULE(a, b)
+
+    @staticmethod
+    def uge(a, b):
+        return _z3.UGE(a, b)
+
+    @staticmethod
+    def eq(a, b):
+        return a == b
+
+    @staticmethod
+    def ite(c, a, b):
+        return _z3.If(c, a, b)
+
+    @staticmethod
+    def implies(a, b):
+        return _z3.Implies(a, b)
+
+    @staticmethod
+    def all_of(*xs):
+        return _z3.And(*xs)
+
+    @staticmethod
+    def any_of(*xs):
+        return _z3.Or(*xs)
+
+
+def _enumerate(domains: dict, constraints, count: int, backend: str = "auto"):
+    """All assignments of `domains` (name -> tuple of ints) that satisfy
+    `constraints(ops, vars) -> list of boolean expressions`, as sorted tuples in
+    the key order of `domains`, at most `count` of them."""
+    names = list(domains)
+    use_z3 = backend == "z3" or (backend == "auto" and _z3 is not None)
+    if use_z3:
+        if _z3 is None:
+            raise RuntimeError("z3 backend requested but z3 is not importable")
+        ops = _Z3Ops
+        vs = {n: _z3.BitVec(n, _Z3Ops.BITS) for n in names}
+        s = _z3.Solver()
+        for n in names:
+            s.add(_z3.Or([vs[n] == v for v in domains[n]]))
+        s.add(*constraints(ops, vs))
+        found = []
+        while len(found) < count and s.check() == _z3.sat:
+            m = s.model()
+            vals = tuple(m[vs[n]].as_long() for n in names)
+            found.append(vals)
+            s.add(_z3.Or([vs[n] != v for n, v in zip(names, vals)]))
+        return sorted(found)
+    found = []
+    for vals in itertools.product(*(domains[n] for n in names)):
+        if all(constraints(_IntOps, dict(zip(names, vals)))):
+            found.append(vals)
+    return sorted(found)[:count]
+
+
+def _satisfiable(domains: dict, constraints, backend: str = "auto") -> bool:
+    return len(_enumerate(domains, constraints, 1, backend)) > 0
+
+
+# ---------------------------------------------------------------------------
+# row-wise (Softmax / RMSNorm)
+# ---------------------------------------------------------------------------
+ROWWISE_DOMAINS = {
+    "tpr": (16, 32, 64, 128, 256, 512, 1024),
+    "rpb": (1, 2, 4, 8, 16),
+    "vec": (4, 8),
+    "mode": (0, 1),
+    "unroll": (1, 2, 4),
+    "hint": (0, 1),
+}
+
+
+def _rowwise_constraints(arch, op: str, M: int, N: int, type_size: int, force_reg: bool):
+    wave = arch.warp_size
+    simds = arch.simds_per_cu
+
+    def build(o, v):
+        tpr, rpb, vec, mode, unroll, hint = (v[k] for k in ROWWISE_DOMAINS)
+        c = o.const
+        n, m = c(N), c(M)
+        threads = tpr * rpb
+        span = tpr * vec
+        chunks = o.udiv(n + span - 1, span)
+        out = [
+            # whole waves, at most one workgroup's worth of lanes
+            o.uge(threads, c(wave)), o.ule(threads, c(arch.max_threads_per_block)),
+            o.eq(o.urem(threads, c(wave)), c(0)),
+            o.eq(o.urem(n, vec), c(0)),
+            o.eq(o.urem(m, rpb), c(0)),
+            # a row keeps every vector lane of its lanes busy at least once
+            o.ule(span, n),
+            # enough workgroups to give every CU at least one
+            o.uge(o.udiv(m, rpb), c(arch.sm_nums)),
+            # cache-hinted accesses are 8 or 16 bytes
+            o.implies(o.eq(hint, c(1)), o.uge(vec * type_size, c(8))),
+        ]
+        # VGPRs of the cached elements + bookkeeping, as in
+        # rowwise_hip.est_regs_per_thread
+        elems = o.ite(o.eq(mode, c(0)), chunks, unroll) * vec
+        if op == "softmax":
+            regs = o.udiv(elems * 9, c(8)) + 12
+        else:
+            regs = o.udiv(elems * 5, c(4)) + 16 + o.udiv(vec, c(2))
+        regs8 = o.udiv(regs + 7, c(8)) * 8
+        waves_per_simd = o.udiv(o.udiv(threads, c(wave)) + (simds - 1), c(simds))
+        out += [
+            o.ule(regs, c(arch.max_arch_vgprs)),
+            o.ule(regs8 * waves_per_simd, c(arch.vgprs_per_simd)),
+            # reg mode is fully unrolled; twopass needs one full loop iteration
+            o.implies(o.eq(mode, c(0)), o.all_of(o.eq(unroll, c(1)), o.ule(chunks, c(32)))),
+            o.implies(o.eq(mode, c(1)), o.ule(unroll, o.udiv(n, span))),
+        ]
+        if force_reg:
+            out.append(o.eq(mode, c(0)))
+        return out
+
+    return build
+
+
+def solve_rowwise(
+    arch,
+    op: str,
+    M: int,
+    N: int,
+    type_size: int = 2,
+    twopass_min_n: int = 16384,
+    count: int = 1024,
+    backend: str = "auto",
+):
+    """
+    Enumerate row-wise (Softmax / RMSNorm) kernel configurations.
+    Args:
+        arch: Arch, the target GPU
+        op: "softmax" or "rmsnorm"
+        M, N: rows and reduced dimension
+        type_size: bytes per element (2 for fp16 / bf16)
+        twopass_min_n: rows at least this long may also be streamed twice
+            (always allowed when no register-cached config fits)
+        count: the maximum number of solutions to find
+    Returns:
+        list of RowConfig
+    """
+    from deca_amd.kernels.rowwise_hip import RowConfig
+
+    reg_only = _rowwise_constraints(arch, op, M, N, type_size, force_reg=True)
+    force_reg = N < twopass_min_n and _satisfiable(ROWWISE_DOMAINS, reg_only, backend)
+    cons = reg_only if force_reg else _rowwise_constraints(arch, op, M, N, type_size, False)
+    return [
+        RowConfig(
+            threads_per_row=tpr, rows_per_block=rpb, vec=vec,
+            mode="twopass" if mode else "reg", unroll=unroll, hint=bool(hint),
+        )
+        for tpr, rpb, vec, mode, unroll, hint in _enumerate(ROWWISE_DOMAINS, cons, count, backend)
+    ]

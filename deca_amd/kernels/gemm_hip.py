@@ -1,0 +1,152 @@
+"""
+FP16 MFMA GEMM (C = A @ B, fp32 accumulation): config type, resource estimates,
+validity rules and the specialisation of the HIP template `csrc/gemm.hip`.
+
+Counterpart of the reference's src/kernels/gemm_tir.py.  Layout: A[M, K],
+B[K, N], C[M, N], all row-major float16.
+
+What changes on CDNA4 (reference mechanism -> here):
+- mma.sync.m16n8k16 (gemm_tir.py:280-290) -> v_mfma_f32_32x32x16_f16; a wave is
+  64 lanes and owns a `warp_m x warp_n` tile made of 32x32 MFMA tiles;
+- ldmatrix / ldmatrix.trans (:262-278) -> ds_read_b128 for A and the transposing
+  ds_read_b64_tr_b16 for the row-major B tile;
+- cp.async ring (:190-199) -> 16-byte global loads staged through VGPRs one
+  K-tile ahead of the MFMAs, into a 1- or 2-deep LDS ring;
+- 128-byte-line XOR swizzle (:14-18) -> chunk swizzles sized for the 64-bank LDS;
+- grouped rasterisation (:159-163) -> the same grouping applied after dealing
+  contiguous tile ranges to the 8 XCDs (each has a private L2);
+- fp16 accumulation (`acc_f16`, `acc_splits`, :52-58) has no MFMA counterpart
+  (the matrix cores always accumulate in fp32) and is not offered.
+"""
+
+from __future__ import annotations
+
+from dataclasses import asdict, dataclass
+
+from deca_amd.kernels.build import (
+    DEFAULT_ARCH, FAST_MATH_OPTIONS, KernelSpec, build_kernel, cached_build, make_spec,
+)
+
+WAVE = 64
+MFMA_M = 32  # v_mfma_f32_32x32x16_f16
+MFMA_K = 16
+MAX_VGPRS = 512  # unified VGPRs (arch + accumulation) per lane at one wave per SIMD
+MAX_LDS = 160 * 1024
+# Padding (halves) of the epilogue staging rows.
+EPI_PAD = 8
+TEMPLATE = "gemm.hip"
+
+
+@dataclass(frozen=True)
+class GemmConfig:
+    BM: int = 256  # workgroup tile rows
+    BN: int = 256  # workgroup tile columns
+    BK: int = 64  # K depth of one pipeline stage
+    warp_m: int = 128  # wave tile rows
+    warp_n: int = 128  # wave tile columns
+    stages: int = 2  # LDS ring depth (1 or 2; global loads are always one tile ahead)
+    raster: int = 8  # workgroup rows per rasterisation group (1: plain row-major order)
+    epi_smem: bool = False  # stage C through LDS for 16-byte stores
+    xcd: bool = True  # deal contiguous tile ranges to the 8 XCDs
+
+    @property
+    def num_warps(self) -> int:
+        return (self.BM // self.warp_m) * (self.BN // self.warp_n)
+
+    @property
+    def threads(self) -> int:
+        return self.num_warps * WAVE
+
+    def as_dict(self):
+        return asdict(self)
+
+    def __str__(self):
+        return (
+            f"{self.BM}x{self.BN}x{self.BK},warp={self.warp_m}x{self.warp_n},"
+            f"stages={self.stages},raster={self.raster},epi_smem={int(self.epi_smem)}"
+            + ("" if self.xcd else ",xcd=0")
+        )
+
+
+def pipeline_smem_bytes(cfg: GemmConfig) -> int:
+    return cfg.stages * (cfg.BM * cfg.BK + cfg.BK * cfg.BN) * 2
+
+
+def epilogue_smem_bytes(cfg: GemmConfig) -> int:
+    return cfg.BM * (cfg.BN + EPI_PAD) * 2 if cfg.epi_smem else 0
+
+
+def smem_bytes(cfg: GemmConfig) -> int:
+    """The epilogue reuses the pipeline buffers once the main loop is done."""
+    return max(pipeline_smem_bytes(cfg), epilogue_smem_bytes(cfg))
+
+
+def est_regs_per_thread(cfg: GemmConfig) -> int:
+    """Unified VGPR estimate per lane: fp32 accumulators (warp_m * warp_n / 64),
+    one set of A / B fragments (4 VGPRs per 32-row tile), the global->LDS
+    staging registers and addressing."""
+    acc = cfg.warp_m * cfg.warp_n // WAVE
+    frags = 4 * (cfg.warp_m // MFMA_M + cfg.warp_n // MFMA_M)
+    staging = (cfg.BM * cfg.BK + cfg.BK * cfg.BN) // 8 // cfg.threads * 4
+    return acc + frags + staging + 40
+
+
+def check_config(cfg: GemmConfig, M: int, N: int, K: int, max_smem: int = MAX_LDS) -> None:
+    assert cfg.stages in (1, 2)
+    assert smem_bytes(cfg) <= max_smem
+    assert cfg.BK in (32, 64)
+    assert cfg.warp_m % MFMA_M == 0 and cfg.warp_n % MFMA_M == 0
+    assert cfg.BM % cfg.warp_m == 0 and cfg.BN % cfg.warp_n == 0
+    assert cfg.BN >= 64
+    assert M % cfg.BM == 0 and N % cfg.BN == 0 and K % cfg.BK == 0
+    assert WAVE <= cfg.threads <= 1024
+    # Every lane issues the same number of 16-byte loads for each operand.
+    assert (cfg.BM * cfg.BK // 8) % cfg.threads == 0
+    assert (cfg.BK * cfg.BN // 8) % cfg.threads == 0
+    assert (M // cfg.BM) % cfg.raster == 0
+    if cfg.xcd:
+        assert ((M // cfg.BM) * (N // cfg.BN)) % 8 == 0
+    if cfg.epi_smem:
+        assert (cfg.BM * cfg.BN // 8) % cfg.threads == 0
+    assert est_regs_per_thread(cfg) <= MAX_VGPRS
+
+
+def make_gemm_tc(M: int, N: int, K: int, cfg: GemmConfig) -> KernelSpec:
+    """Specialised kernel: 1-D grid of (M/BM)*(N/BN) workgroups of `threads`
+    lanes (reference: gemm_tir.py:156), static LDS."""
+    check_config(cfg, M, N, K)
+    defines = {
+        "DECA_M": M, "DECA_N": N, "DECA_K": K,
+        "DECA_BM": cfg.BM, "DECA_BN": cfg.BN, "DECA_BK": cfg.BK,
+        "DECA_WM": cfg.warp_m, "DECA_WN": cfg.warp_n,
+        "DECA_STAGES": cfg.stages, "DECA_RASTER": cfg.raster,
+        "DECA_EPI_LDS": int(cfg.epi_smem), "DECA_XCD": int(cfg.xcd),
+    }
+    return make_spec(
+        TEMPLATE, defines, grid=((M // cfg.BM) * (N // cfg.BN), 1, 1), block=(cfg.threads, 1, 1),
+        nargs=3, options=FAST_MATH_OPTIONS, meta={"cfg": str(cfg)},
+    )
+
+
+GEMM_HIPCC_OPTIONS = FAST_MATH_OPTIONS
+
+
+def build_gemm_tc(spec: KernelSpec, target: str | None = None, dump_dir: str | None = None):
+    """Compiles (or takes from the in-tree cache) and loads the kernel;
+    `dump_dir` keeps the generated ISA for inspection."""
+    import os
+
+    from deca_amd.driver.driver import load_kernel
+
+    arch = target or DEFAULT_ARCH
+    if dump_dir:
+        path = build_kernel(spec, arch, os.path.join(dump_dir, f"gemm_{spec.key()}.hsaco"), dump_dir)
+    else:
+        path = cached_build(spec, arch)
+    return load_kernel(spec, path)
+
+
+def build_gemm_tc_to_file(shape, cfg: GemmConfig, arch: str, path: str) -> str:
+    """Builds in a worker process (no GPU context needed) and writes a code object."""
+    M, N, K = shape
+    return build_kernel(make_gemm_tc(M, N, K, cfg), arch, path)

@@ -1,6 +1,7 @@
 """Kernel specialisations the GPU tests use, listed in one place so that the
 build step can compile all of them ahead of the GPU run."""
 
+from deca_amd.kernels.gemm_hip import GemmConfig, make_gemm_tc
 from deca_amd.kernels.rowwise_hip import RowConfig, make_rowwise
 
 # (op, M, N, dtype, cfg)
@@ -51,5 +52,33 @@ def rowwise_specs(eps: float = 1e-6):
     return [make_rowwise(op, M, N, dt, cfg, eps) for op, M, N, dt, cfg in ROWWISE_CASES + ROWWISE_FULL]
 
 
+# (M, N, K, cfg): sizes the CPU checker finishes in seconds
+GEMM_CASES = [
+    (512, 512, 512, GemmConfig(256, 256, 64, 128, 128, 2, 1, False, False)),
+    (512, 512, 512, GemmConfig(256, 256, 64, 128, 128, 2, 2, True, False)),
+    (512, 1024, 256, GemmConfig(256, 256, 32, 128, 128, 2, 2, False, True)),
+    (512, 512, 512, GemmConfig(256, 256, 64, 128, 64, 2, 1, False, False)),
+    (512, 512, 512, GemmConfig(256, 256, 64, 64, 128, 2, 1, True, False)),
+    (512, 512, 512, GemmConfig(128, 128, 64, 64, 64, 2, 4, False, True)),
+    (512, 512, 512, GemmConfig(128, 128, 32, 64, 32, 1, 4, True, True)),
+    (384, 640, 1088, GemmConfig(128, 128, 64, 64, 64, 2, 1, False, False)),
+    (512, 512, 2048, GemmConfig(128, 256, 64, 64, 128, 2, 2, False, True)),
+    (512, 256, 192, GemmConfig(256, 128, 64, 128, 64, 1, 1, True, False)),
+    (256, 256, 64, GemmConfig(64, 64, 64, 32, 32, 2, 1, False, False)),
+    (128, 192, 32, GemmConfig(64, 64, 32, 32, 64, 1, 2, False, False)),
+    (1024, 1024, 512, GemmConfig(256, 256, 64, 128, 128, 2, 4, False, True)),
+]
+
+# Full-size shapes: checked on a sample of rows against the CPU checker.
+GEMM_FULL = [
+    (4096, 4096, 4096, GemmConfig(256, 256, 64, 128, 128, 2, 8, False, True)),
+    (8192, 8192, 8192, GemmConfig(256, 256, 64, 128, 128, 2, 8, False, True)),
+]
+
+
+def gemm_specs():
+    return [make_gemm_tc(M, N, K, cfg) for M, N, K, cfg in GEMM_CASES + GEMM_FULL]
+
+
 def all_specs():
-    return rowwise_specs()
+    return rowwise_specs() + gemm_specs()
