@@ -11,11 +11,16 @@
 //   DECA_EPI_LDS  1: stage C through LDS for 16-byte stores
 //   DECA_XCD      1: remap workgroup ids so that each of the 8 XCDs (private L2)
 //                 owns a contiguous slab of tiles
+//   DECA_DIRECT   1: global -> LDS loads that bypass the VGPRs, ring of
+//                 DECA_STAGES (2..4) tiles; 0: loads staged through VGPRs one
+//                 tile ahead, ring of 1 or 2 tiles
 //
 // Data path (what the reference does with cp.async + ldmatrix + mma.sync,
 // gemm_tir.py:190-334):
-//   global -> VGPR (16-byte loads, issued one K-tile ahead) -> LDS
-//   (ds_write_b128, XOR-swizzled chunks) -> fragments: A by ds_read_b128
+//   global -> LDS, either directly (global_load_lds_dwordx4, asynchronous,
+//   counted by vmcnt like cp.async groups) or through VGPRs (16-byte loads
+//   issued one K-tile ahead, then ds_write_b128), XOR-swizzled chunks
+//   -> fragments, double buffered in registers one k-step ahead: A by ds_read_b128
 //   (8 consecutive k per lane), B by ds_read_b64_tr_b16 (transposing read, so
 //   the row-major [k][n] tile feeds the k-packed MFMA operand directly)
 //   -> MFMA 32x32x16 with the operand roles swapped (B fragment as the first
@@ -63,7 +68,8 @@ static_assert(BM % WM == 0 && BN % WN == 0 && WM % 32 == 0 && WN % 32 == 0, "wav
 static_assert(BK % 16 == 0 && (CPR_A == 4 || CPR_A == 8), "BK must be 32 or 64");
 static_assert(A_CHUNKS % NT == 0 && B_CHUNKS % NT == 0, "loader coverage");
 static_assert(NT >= 64 && NT <= 1024, "workgroup size");
-static_assert(STAGES == 1 || STAGES == 2, "LDS ring depth");
+static_assert(STAGES >= 1 && STAGES <= 4, "LDS ring depth");
+static_assert(DECA_DIRECT == 0 || STAGES >= 2, "the direct-to-LDS ring needs two slots");
 static_assert(GM % DECA_RASTER == 0, "raster group must divide the workgroup rows");
 static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
 static_assert(CPR_B >= 8, "BN >= 64");
@@ -74,6 +80,8 @@ typedef short short4v __attribute__((ext_vector_type(4)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) short4v* lds_s4_ptr;
+typedef const __attribute__((address_space(1))) void* gptr;
+typedef __attribute__((address_space(3))) void* lptr;
 
 // ---- LDS layouts -----------------------------------------------------------
 // A tile: [BM][BK] halves, k contiguous; 16-byte chunk c of row r sits at chunk
@@ -117,12 +125,181 @@ deca_main(const _Float16* __restrict__ A, const _Float16* __restrict__ B,
   const int bm = (lin / GROUP) * DECA_RASTER + (lin % GROUP) % DECA_RASTER;
   const int bn = (lin % GROUP) / DECA_RASTER;
 
-  // ---- global -> register staging -------------------------------------------
-  u32x4 a_stage[A_IT];
-  u32x4 b_stage[B_IT];
   const _Float16* a_gbase = A + static_cast<size_t>(bm) * BM * K_;
   const _Float16* b_gbase = B + static_cast<size_t>(bn) * BN;
 
+  // ---- accumulators and fragment addressing -----------------------------------
+  floatx16 acc[MT][NTL];
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int j = 0; j < NTL; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+  const int l32 = lane & 31;
+  const int khalf = lane >> 5;
+  // transposing B read: 16-lane block tb, lane ti in the block supplies the
+  // address of row k0 + ti/4, columns n0 + 4*(ti%4) .. +3 and receives, for its
+  // column n0 + ti, the four rows k0 .. k0+3
+  const int tb = lane >> 4, ti = lane & 15;
+  const int b_n_off = 16 * (tb & 1) + 4 * (ti & 3);  // + wn0 + nt * 32
+  const int b_k_off = (tb >> 1) * 8 + (ti >> 2);     // + ks * 16 + r * 4
+
+  // Fragments of k-step `ks` of the tile in ring slot `slot`.
+  auto load_frags = [&](half8 (&af)[MT], half8 (&bf)[NTL], int slot, int ks) {
+    const unsigned char* a_lds = lds + slot * A_STAGE_BYTES;
+    const unsigned char* b_lds = lds + STAGES * A_STAGE_BYTES + slot * B_STAGE_BYTES;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const int row = wm0 + mt * 32 + l32;
+      af[mt] = *reinterpret_cast<const half8*>(a_lds + a_chunk_slot(row, ks * 2 + khalf) * 16);
+    }
+#pragma unroll
+    for (int nt = 0; nt < NTL; ++nt) {
+      const int n = wn0 + nt * 32 + b_n_off;
+      half4 h[2];
+#pragma unroll
+      for (int r = 0; r < 2; ++r) {
+        const int k = ks * 16 + r * 4 + b_k_off;
+        const unsigned char* p = b_lds + b_chunk_slot(k, n >> 3) * 16 + ((n >> 2) & 1) * 8;
+        h[r] = __builtin_bit_cast(half4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4_ptr)(p)));
+      }
+      bf[nt] = __builtin_shufflevector(h[0], h[1], 0, 1, 2, 3, 4, 5, 6, 7);
+    }
+  };
+  // Operand roles are swapped (B fragment first) so that a lane's four
+  // consecutive accumulator registers are four consecutive n of one row of C.
+  auto mfma_step = [&](const half8 (&af)[MT], const half8 (&bf)[NTL]) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < NTL; ++nt)
+        acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[nt], af[mt], acc[mt][nt], 0, 0, 0);
+  };
+
+  // Scheduling pattern of one k-step: the LDS reads of the next fragments are
+  // issued one per MFMA, so that they hide under the matrix pipe instead of
+  // being grouped after it (mask 0x100 = DS read, 0x008 = MFMA).
+  auto interleave_reads_with_mfma = [&]() {
+    constexpr int READS = MT + 2 * NTL;
+    constexpr int MFMAS = MT * NTL;
+    constexpr int PAIRS = READS < MFMAS ? READS : MFMAS;
+#pragma unroll
+    for (int i = 0; i < PAIRS; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    if (READS > PAIRS) __builtin_amdgcn_sched_group_barrier(0x100, READS - PAIRS, 0);
+    if (MFMAS > PAIRS) __builtin_amdgcn_sched_group_barrier(0x008, MFMAS - PAIRS, 0);
+  };
+
+  half8 af0[MT], bf0[NTL], af1[MT], bf1[NTL];
+
+#if DECA_DIRECT
+  // ---- main loop: direct-to-LDS ring ---------------------------------------------
+  // Tile kt lives in ring slot kt % STAGES.  Each lane issues LOADS 16-byte
+  // global->LDS loads per tile; the hardware writes lane L's data to
+  // (wave-uniform base) + L * 16, so the swizzle is applied by choosing which
+  // global chunk each lane fetches.
+  constexpr int LOADS = A_IT + B_IT;
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  const unsigned lds_u = static_cast<unsigned>(reinterpret_cast<size_t>((lptr)lds));
+  // Byte offset of each lane's chunk from the tile's (wave-uniform) origin.
+  unsigned a_voff[A_IT], b_voff[B_IT];
+#pragma unroll
+  for (int it = 0; it < A_IT; ++it) {
+    const int sidx = it * NT + tid;
+    const int row = sidx / CPR_A;
+    const int c = (sidx % CPR_A) ^ ((row / (16 / CPR_A)) % CPR_A);
+    a_voff[it] = static_cast<unsigned>(row * K_ + c * 8) * 2u;
+  }
+#pragma unroll
+  for (int it = 0; it < B_IT; ++it) {
+    const int sidx = it * NT + tid;
+    const int k = sidx / CPR_B;
+    const int c = (sidx % CPR_B) ^ (((k & 3) << 2) & (CPR_B - 1));
+    b_voff[it] = static_cast<unsigned>(k * N_ + c * 8) * 2u;
+  }
+  static_assert(static_cast<long long>(BM) * K_ * 2 < (1ll << 32) &&
+                static_cast<long long>(BK) * N_ * 2 < (1ll << 32), "32-bit lane offsets");
+  // The load is written as inline assembly so that the compiler's wait-count
+  // insertion does not see an LDS write and force vmcnt(0) before every LDS
+  // read; the waits are explicit (DECA_WAIT_VMCNT) and paired with a barrier.
+  // The "memory" clobber keeps LDS reads from moving across the issue point.
+  auto dma16 = [&](const _Float16* origin, unsigned voff, unsigned lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(voff), "s"(origin), "s"(lds_addr)
+                 : "memory");
+  };
+  auto issue_tile = [&](int kt, int slot) {
+    const _Float16* a_origin = a_gbase + kt * BK;
+    const _Float16* b_origin = b_gbase + static_cast<size_t>(kt) * BK * N_;
+    const unsigned a_dst = lds_u + slot * A_STAGE_BYTES + wave_u * 1024;
+    const unsigned b_dst = lds_u + STAGES * A_STAGE_BYTES + slot * B_STAGE_BYTES + wave_u * 1024;
+#pragma unroll
+    for (int it = 0; it < A_IT; ++it) dma16(a_origin, a_voff[it], a_dst + it * NT * 16);
+#pragma unroll
+    for (int it = 0; it < B_IT; ++it) dma16(b_origin, b_voff[it], b_dst + it * NT * 16);
+  };
+  // s_waitcnt on the vector-memory counter only (gfx9 encoding: vmcnt in bits
+  // 3:0 and 15:14, expcnt 6:4 and lgkmcnt 11:8 left at "no wait").
+#define DECA_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (((n) >> 4) << 14) | 0x0F70)
+  constexpr int PENDING = (STAGES - 2) * LOADS;  // loads that may stay in flight
+  static_assert(PENDING <= 63, "vmcnt holds 6 bits");
+  static_assert(NK >= STAGES, "K too short for the ring");
+
+#pragma unroll
+  for (int s = 0; s < STAGES - 1; ++s) issue_tile(s, s);
+  DECA_WAIT_VMCNT(PENDING);
+  __builtin_amdgcn_s_barrier();
+  load_frags(af0, bf0, 0, 0);
+
+  int slot = 0;
+  for (int kt = 0; kt < NK; ++kt) {
+    const bool more = kt + STAGES - 1 < NK;
+    int fill = slot + STAGES - 1;
+    if (fill >= STAGES) fill -= STAGES;
+    if (more) issue_tile(kt + STAGES - 1, fill);
+    int next = slot + 1;
+    if (next == STAGES) next = 0;
+    // k-steps 0 .. KS-2: fragments of step ks+1 are fetched under the MFMAs of ks
+#pragma unroll
+    for (int ks = 0; ks < KS - 1; ++ks) {
+      if (ks & 1) {
+        load_frags(af0, bf0, slot, ks + 1);
+        mfma_step(af1, bf1);
+      } else {
+        load_frags(af1, bf1, slot, ks + 1);
+        mfma_step(af0, bf0);
+      }
+      interleave_reads_with_mfma();
+    }
+    // Tile kt+1 must have landed for every lane of the workgroup, and every
+    // wave must be done reading slot `slot` before the next iteration refills it.
+    if (more) {
+      DECA_WAIT_VMCNT(PENDING);
+    } else {
+      DECA_WAIT_VMCNT(0);
+    }
+    // all of this wave's LDS reads of slot `slot` have returned
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0) only
+    __builtin_amdgcn_s_barrier();
+    if (kt + 1 < NK) {
+      if ((KS - 1) & 1) load_frags(af0, bf0, next, 0);
+      else load_frags(af1, bf1, next, 0);
+    }
+    if ((KS - 1) & 1) mfma_step(af1, bf1);
+    else mfma_step(af0, bf0);
+    if (kt + 1 < NK) interleave_reads_with_mfma();
+    slot = next;
+  }
+  static_assert(KS % 2 == 0, "fragment double buffer assumes an even number of k-steps");
+#else
+  // ---- main loop: VGPR-staged ring -------------------------------------------------
+  u32x4 a_stage[A_IT];
+  u32x4 b_stage[B_IT];
   auto load_global = [&](int kt) {
 #pragma unroll
     for (int it = 0; it < A_IT; ++it) {
@@ -153,65 +330,28 @@ deca_main(const _Float16* __restrict__ A, const _Float16* __restrict__ B,
       *reinterpret_cast<u32x4*>(b_lds + b_chunk_slot(id / CPR_B, id % CPR_B) * 16) = b_stage[it];
     }
   };
-
-  // ---- fragments --------------------------------------------------------------
-  floatx16 acc[MT][NTL];
-#pragma unroll
-  for (int i = 0; i < MT; ++i)
-#pragma unroll
-    for (int j = 0; j < NTL; ++j)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
-
-  const int l32 = lane & 31;
-  const int khalf = lane >> 5;
-  // transposing B read: 16-lane block b, lane i in the block
-  const int tb = lane >> 4, ti = lane & 15;
-  const int b_n_off = 16 * (tb & 1) + 4 * (ti & 3);  // + wn0 + nt * 32
-  const int b_k_off = (tb >> 1) * 8 + (ti >> 2);     // + ks * 16 + r * 4
-
   auto compute = [&](int slot) {
-    const unsigned char* a_lds = lds + slot * A_STAGE_BYTES;
-    const unsigned char* b_lds = lds + STAGES * A_STAGE_BYTES + slot * B_STAGE_BYTES;
+    load_frags(af0, bf0, slot, 0);
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      half8 af[MT];
-      half8 bf[NTL];
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        const int row = wm0 + mt * 32 + l32;
-        af[mt] = *reinterpret_cast<const half8*>(a_lds + a_chunk_slot(row, ks * 2 + khalf) * 16);
+      if (ks & 1) {
+        if (ks + 1 < KS) load_frags(af0, bf0, slot, ks + 1);
+        mfma_step(af1, bf1);
+      } else {
+        if (ks + 1 < KS) load_frags(af1, bf1, slot, ks + 1);
+        mfma_step(af0, bf0);
       }
-#pragma unroll
-      for (int nt = 0; nt < NTL; ++nt) {
-        const int n = wn0 + nt * 32 + b_n_off;
-        half4 h[2];
-#pragma unroll
-        for (int r = 0; r < 2; ++r) {
-          const int k = ks * 16 + r * 4 + b_k_off;
-          const unsigned char* p = b_lds + b_chunk_slot(k, n >> 3) * 16 + ((n >> 2) & 1) * 8;
-          h[r] = __builtin_bit_cast(half4,
-                                    __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4_ptr)(p)));
-        }
-        bf[nt] = __builtin_shufflevector(h[0], h[1], 0, 1, 2, 3, 4, 5, 6, 7);
-      }
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int nt = 0; nt < NTL; ++nt)
-          acc[mt][nt] =
-              __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[nt], af[mt], acc[mt][nt], 0, 0, 0);
     }
   };
+  static_assert(STAGES <= 2, "the VGPR-staged ring is 1 or 2 deep");
 
-  // ---- main loop ---------------------------------------------------------------
   load_global(0);
   store_lds(0);
   __syncthreads();
 #if STAGES == 2
-  // Steady state: the loads of tile kt+1 are in flight while tile kt is
-  // multiplied; one barrier per K-tile.  The last tile is peeled so that the
-  // prefetch is unconditional inside the loop.
+  // The loads of tile kt+1 are in flight while tile kt is multiplied; one
+  // barrier per K-tile.  The last tile is peeled so that the prefetch is
+  // unconditional inside the loop.
   for (int kt = 0; kt < NK - 1; ++kt) {
     const int slot = kt & 1;
     load_global(kt + 1);
@@ -230,6 +370,7 @@ deca_main(const _Float16* __restrict__ A, const _Float16* __restrict__ B,
   }
   compute(0);
 #endif
+#endif  // DECA_DIRECT
 #if DECA_EPI_LDS
   __syncthreads();
 #endif

@@ -44,10 +44,11 @@ class GemmConfig:
     BK: int = 64  # K depth of one pipeline stage
     warp_m: int = 128  # wave tile rows
     warp_n: int = 128  # wave tile columns
-    stages: int = 2  # LDS ring depth (1 or 2; global loads are always one tile ahead)
+    stages: int = 2  # LDS ring depth: 2..4 with direct loads, 1..2 with VGPR staging
     raster: int = 8  # workgroup rows per rasterisation group (1: plain row-major order)
     epi_smem: bool = False  # stage C through LDS for 16-byte stores
     xcd: bool = True  # deal contiguous tile ranges to the 8 XCDs
+    direct: bool = True  # global -> LDS loads that bypass the VGPRs (else VGPR-staged)
 
     @property
     def num_warps(self) -> int:
@@ -65,6 +66,7 @@ class GemmConfig:
             f"{self.BM}x{self.BN}x{self.BK},warp={self.warp_m}x{self.warp_n},"
             f"stages={self.stages},raster={self.raster},epi_smem={int(self.epi_smem)}"
             + ("" if self.xcd else ",xcd=0")
+            + ("" if self.direct else ",direct=0")
         )
 
 
@@ -86,13 +88,16 @@ def est_regs_per_thread(cfg: GemmConfig) -> int:
     one set of A / B fragments (4 VGPRs per 32-row tile), the global->LDS
     staging registers and addressing."""
     acc = cfg.warp_m * cfg.warp_n // WAVE
-    frags = 4 * (cfg.warp_m // MFMA_M + cfg.warp_n // MFMA_M)
-    staging = (cfg.BM * cfg.BK + cfg.BK * cfg.BN) // 8 // cfg.threads * 4
-    return acc + frags + staging + 40
+    frags = 4 * (cfg.warp_m // MFMA_M + cfg.warp_n // MFMA_M)  # one of the two sets
+    chunks = (cfg.BM * cfg.BK + cfg.BK * cfg.BN) // 8 // cfg.threads
+    # direct loads keep one offset register per chunk, staged loads four data registers
+    staging = chunks if cfg.direct else chunks * 4
+    return acc + 2 * frags + staging + 40
 
 
 def check_config(cfg: GemmConfig, M: int, N: int, K: int, max_smem: int = MAX_LDS) -> None:
-    assert cfg.stages in (1, 2)
+    assert cfg.stages in ((2, 3, 4) if cfg.direct else (1, 2))
+    assert K // cfg.BK >= cfg.stages
     assert smem_bytes(cfg) <= max_smem
     assert cfg.BK in (32, 64)
     assert cfg.warp_m % MFMA_M == 0 and cfg.warp_n % MFMA_M == 0
@@ -121,6 +126,7 @@ def make_gemm_tc(M: int, N: int, K: int, cfg: GemmConfig) -> KernelSpec:
         "DECA_WM": cfg.warp_m, "DECA_WN": cfg.warp_n,
         "DECA_STAGES": cfg.stages, "DECA_RASTER": cfg.raster,
         "DECA_EPI_LDS": int(cfg.epi_smem), "DECA_XCD": int(cfg.xcd),
+        "DECA_DIRECT": int(cfg.direct),
     }
     return make_spec(
         TEMPLATE, defines, grid=((M // cfg.BM) * (N // cfg.BN), 1, 1), block=(cfg.threads, 1, 1),

@@ -54,25 +54,31 @@ def rowwise_specs(eps: float = 1e-6):
 
 # (M, N, K, cfg): sizes the CPU checker finishes in seconds
 GEMM_CASES = [
-    (512, 512, 512, GemmConfig(256, 256, 64, 128, 128, 2, 1, False, False)),
-    (512, 512, 512, GemmConfig(256, 256, 64, 128, 128, 2, 2, True, False)),
-    (512, 1024, 256, GemmConfig(256, 256, 32, 128, 128, 2, 2, False, True)),
-    (512, 512, 512, GemmConfig(256, 256, 64, 128, 64, 2, 1, False, False)),
-    (512, 512, 512, GemmConfig(256, 256, 64, 64, 128, 2, 1, True, False)),
-    (512, 512, 512, GemmConfig(128, 128, 64, 64, 64, 2, 4, False, True)),
-    (512, 512, 512, GemmConfig(128, 128, 32, 64, 32, 1, 4, True, True)),
-    (384, 640, 1088, GemmConfig(128, 128, 64, 64, 64, 2, 1, False, False)),
-    (512, 512, 2048, GemmConfig(128, 256, 64, 64, 128, 2, 2, False, True)),
-    (512, 256, 192, GemmConfig(256, 128, 64, 128, 64, 1, 1, True, False)),
-    (256, 256, 64, GemmConfig(64, 64, 64, 32, 32, 2, 1, False, False)),
-    (128, 192, 32, GemmConfig(64, 64, 32, 32, 64, 1, 2, False, False)),
-    (1024, 1024, 512, GemmConfig(256, 256, 64, 128, 128, 2, 4, False, True)),
+    # direct-to-LDS ring: (BM, BN, BK, wm, wn, stages, raster, epi_smem, xcd, direct)
+    (512, 512, 512, GemmConfig(256, 256, 64, 128, 128, 2, 1, False, False, True)),
+    (512, 512, 512, GemmConfig(256, 256, 32, 128, 128, 3, 2, True, False, True)),
+    (512, 1024, 256, GemmConfig(256, 256, 32, 128, 128, 4, 2, False, True, True)),
+    (512, 512, 512, GemmConfig(256, 256, 64, 128, 64, 2, 1, False, False, True)),
+    (512, 512, 512, GemmConfig(256, 256, 32, 64, 128, 4, 1, True, False, True)),
+    (512, 512, 512, GemmConfig(128, 128, 64, 64, 64, 3, 4, False, True, True)),
+    (512, 512, 512, GemmConfig(128, 128, 32, 64, 32, 4, 4, True, True, True)),
+    (384, 640, 1088, GemmConfig(128, 128, 64, 64, 64, 2, 1, False, False, True)),
+    (512, 512, 2048, GemmConfig(128, 256, 64, 64, 128, 3, 2, False, True, True)),
+    (256, 256, 128, GemmConfig(64, 64, 64, 32, 32, 2, 1, False, False, True)),
+    (128, 192, 64, GemmConfig(64, 64, 32, 32, 64, 2, 2, False, False, True)),
+    (1024, 1024, 512, GemmConfig(256, 256, 32, 128, 128, 3, 4, False, True, True)),
+    # VGPR-staged ring
+    (512, 512, 512, GemmConfig(256, 256, 64, 128, 128, 2, 1, False, False, False)),
+    (512, 1024, 256, GemmConfig(256, 256, 32, 128, 128, 2, 2, True, True, False)),
+    (512, 512, 512, GemmConfig(128, 128, 32, 64, 32, 1, 4, True, True, False)),
+    (512, 256, 192, GemmConfig(256, 128, 64, 128, 64, 1, 1, True, False, False)),
+    (128, 192, 32, GemmConfig(64, 64, 32, 32, 64, 1, 2, False, False, False)),
 ]
 
 # Full-size shapes: checked on a sample of rows against the CPU checker.
 GEMM_FULL = [
-    (4096, 4096, 4096, GemmConfig(256, 256, 64, 128, 128, 2, 8, False, True)),
-    (8192, 8192, 8192, GemmConfig(256, 256, 64, 128, 128, 2, 8, False, True)),
+    (4096, 4096, 4096, GemmConfig(256, 256, 64, 128, 128, 2, 8, False, True, True)),
+    (8192, 8192, 8192, GemmConfig(256, 256, 32, 128, 128, 3, 8, False, True, True)),
 ]
 
 
