@@ -1,0 +1,337 @@
+// FlashAttention forward, O = softmax(scale * Q K^T [+ causal mask]) V, for gfx950.
+// Q, K, V, O are contiguous [B, H, S, D] float16; fp32 scores and accumulators.
+//
+// One code object per (shape, FAConfig); the DECA_* macros are compile-time
+// constants supplied by kernels/flash_attn_hip.py, as the reference bakes shape
+// and config into each generated kernel (src/kernels/flash_attn_tir.py:83-137).
+//
+//   DECA_B/H/SQ/SKV/D   problem          DECA_BR   query rows per workgroup
+//   DECA_BC             key/value rows per step
+//   DECA_NW             waves per workgroup (each owns BR / NW query rows)
+//   DECA_STAGES         K/V LDS ring depth (1 or 2)
+//   DECA_CAUSAL         1: key j visible to query i iff j <= i (SQ == SKV)
+//   DECA_SCALE          softmax scale
+//
+// The problem is computed transposed, which is what makes the two MFMA
+// products chain without a layout change on CDNA:
+//   S^T = K Q^T   first operand K rows (32 keys x 16 d, ds_read_b128),
+//                 second operand Q (32 queries x 16 d, kept in VGPRs);
+//                 a lane then holds ONE query column (lane % 32) and 16 key
+//                 rows per 32-key block, so the row max / row sum of the online
+//                 softmax are in-lane reductions plus one exchange with lane^32;
+//   O^T = V^T P^T first operand V^T (32 d x 16 keys, transposing
+//                 ds_read_b64_tr_b16 of the row-major V tile), second operand
+//                 P^T taken straight from the S^T accumulator registers (its
+//                 register order is, by construction, the k-packed operand
+//                 order once the matching key rows are chosen for V).
+// The per-query rescale factor is a per-lane scalar.  K/V tiles arrive by
+// global->LDS loads one step ahead (ring of DECA_STAGES slots).
+//
+// Numerics follow src/kernels/flash_attn_tir.py:379-458: unscaled fp32 S; mask
+// value -1e30 on tiles crossing the diagonal only; m' = max(m, rowmax S);
+// alpha = exp2((m - m') * sl2); p = exp2(S * sl2 - m' * sl2), sl2 = scale * log2e;
+// l = l * alpha + sum p (fp32 p); P = fp16(p) feeds the second product;
+// O = O * alpha + P V; final O / l -> fp16.
+#include <hip/hip_runtime.h>
+
+#ifndef DECA_BR
+#error "flash_attn.hip is a template: define the DECA_* macros"
+#endif
+
+#define D_ DECA_D
+#define BR DECA_BR
+#define BC DECA_BC
+#define NW DECA_NW
+#define STAGES DECA_STAGES
+
+constexpr int NT = NW * 64;
+constexpr int WQ = BR / NW;       // query rows per wave
+constexpr int MQ = WQ / 32;       // 32-query MFMA tiles per wave
+constexpr int KT = BC / 32;       // 32-key blocks per step (S^T row tiles)
+constexpr int DK = D_ / 16;       // k-steps of S^T = K Q^T
+constexpr int DT = D_ / 32;       // 32-d blocks of O^T
+constexpr int KK = BC / 16;       // k-steps of O^T = V^T P^T
+constexpr int CPR = D_ / 8;       // 16-byte chunks per K/V row
+constexpr int TILE_CHUNKS = BC * CPR;
+constexpr int TILE_BYTES = TILE_CHUNKS * 16;
+constexpr int KV_IT = TILE_CHUNKS / NT;
+constexpr int NKV = DECA_SKV / BC;
+constexpr int LDS_BYTES = 2 * STAGES * TILE_BYTES;
+constexpr float LOG2E = 1.4426950408889634f;
+constexpr float NEG_INF = -1e30f;
+constexpr float SL2 = static_cast<float>(DECA_SCALE) * LOG2E;
+
+static_assert(D_ % 64 == 0, "head dim must be a multiple of 64");
+static_assert(BR % (32 * NW) == 0, "each wave owns a multiple of 32 query rows");
+static_assert(BC % 32 == 0, "BC must be a multiple of 32");
+static_assert(DECA_SQ % BR == 0 && DECA_SKV % BC == 0, "tiles must divide the sequences");
+static_assert(TILE_CHUNKS % NT == 0, "loader coverage");
+static_assert(STAGES == 1 || STAGES == 2, "K/V ring depth");
+static_assert(!DECA_CAUSAL || DECA_SQ == DECA_SKV, "causal needs S_q == S_kv");
+static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
+static_assert(2 * KV_IT <= 63, "vmcnt holds 6 bits");
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef short short4v __attribute__((ext_vector_type(4)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef __attribute__((address_space(3))) short4v* lds_s4_ptr;
+typedef __attribute__((address_space(3))) void* lptr;
+
+// K tile [BC][D]: 16 consecutive rows at one logical chunk must land on 16
+// different 16-byte bank groups of the 256-byte bank window.
+__device__ __forceinline__ int k_chunk_slot(int row, int c) {
+  constexpr int ROWS_PER_WINDOW = (16 / CPR) > 0 ? (16 / CPR) : 1;
+  constexpr int MASK = (CPR < 16 ? CPR : 16) - 1;
+  return row * CPR + (c ^ ((row / ROWS_PER_WINDOW) & MASK));
+}
+// V tile [BC][D]: the 4 key rows of one transposing read are rotated onto
+// different 64-byte groups.
+__device__ __forceinline__ int v_chunk_slot(int row, int c) {
+  return row * CPR + (c ^ (((row & 3) << 2) & (CPR - 1)));
+}
+
+#define DECA_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (((n) >> 4) << 14) | 0x0F70)
+
+extern "C" __global__ void __launch_bounds__(NT)
+deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
+          const _Float16* __restrict__ V, _Float16* __restrict__ O) {
+  __shared__ __attribute__((aligned(16))) unsigned char lds[LDS_BYTES];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  const int l32 = lane & 31;
+  const int half = lane >> 5;
+  const int bh = blockIdx.y;
+#if DECA_CAUSAL
+  // Query tiles near the end see the most keys; schedule them first
+  // (flash_attn_tir.py:152-156).
+  const int qt = (DECA_SQ / BR - 1) - static_cast<int>(blockIdx.x);
+  const int nkv = ((qt + 1) * BR + BC - 1) / BC;
+#else
+  const int qt = blockIdx.x;
+  const int nkv = NKV;
+#endif
+  const _Float16* q_base = Q + (static_cast<size_t>(bh) * DECA_SQ + qt * BR + wave * WQ) * D_;
+  const _Float16* k_base = K + static_cast<size_t>(bh) * DECA_SKV * D_;
+  const _Float16* v_base = V + static_cast<size_t>(bh) * DECA_SKV * D_;
+  _Float16* o_base = O + (static_cast<size_t>(bh) * DECA_SQ + qt * BR + wave * WQ) * D_;
+
+  // ---- K/V tile loads: global -> LDS, asynchronous ------------------------------
+  const unsigned lds_u = static_cast<unsigned>(reinterpret_cast<size_t>((lptr)lds));
+  unsigned k_voff[KV_IT], v_voff[KV_IT];
+#pragma unroll
+  for (int it = 0; it < KV_IT; ++it) {
+    const int sidx = it * NT + tid;
+    const int row = sidx / CPR, cs = sidx % CPR;
+    constexpr int ROWS_PER_WINDOW = (16 / CPR) > 0 ? (16 / CPR) : 1;
+    constexpr int MASK = (CPR < 16 ? CPR : 16) - 1;
+    const int ck = cs ^ ((row / ROWS_PER_WINDOW) & MASK);
+    const int cv = cs ^ (((row & 3) << 2) & (CPR - 1));
+    k_voff[it] = static_cast<unsigned>(row * D_ + ck * 8) * 2u;
+    v_voff[it] = static_cast<unsigned>(row * D_ + cv * 8) * 2u;
+  }
+  // Inline assembly keeps the compiler's wait-count insertion from forcing
+  // vmcnt(0) before every LDS read; waits are explicit and paired with barriers.
+  auto dma16 = [&](const _Float16* origin, unsigned voff, unsigned lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(voff), "s"(origin), "s"(lds_addr)
+                 : "memory");
+  };
+  auto issue_tile = [&](int j, int slot) {
+    const _Float16* k_origin = k_base + static_cast<size_t>(j) * BC * D_;
+    const _Float16* v_origin = v_base + static_cast<size_t>(j) * BC * D_;
+    const unsigned k_dst = lds_u + slot * TILE_BYTES + wave_u * 1024;
+    const unsigned v_dst = lds_u + (STAGES + slot) * TILE_BYTES + wave_u * 1024;
+#pragma unroll
+    for (int it = 0; it < KV_IT; ++it) dma16(k_origin, k_voff[it], k_dst + it * NT * 16);
+#pragma unroll
+    for (int it = 0; it < KV_IT; ++it) dma16(v_origin, v_voff[it], v_dst + it * NT * 16);
+  };
+
+  issue_tile(0, 0);
+
+  // ---- Q fragments: VGPR resident for the whole kernel ----------------------------
+  // lane (q = lane % 32, half): 8 consecutive d at ks * 16 + half * 8
+  half8 qf[MQ][DK];
+#pragma unroll
+  for (int mq = 0; mq < MQ; ++mq)
+#pragma unroll
+    for (int ks = 0; ks < DK; ++ks)
+      qf[mq][ks] = *reinterpret_cast<const half8*>(q_base + (mq * 32 + l32) * D_ + ks * 16 + half * 8);
+
+  floatx16 o_acc[DT][MQ];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int mq = 0; mq < MQ; ++mq)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) o_acc[dt][mq][e] = 0.0f;
+  float m_i[MQ], l_i[MQ];
+#pragma unroll
+  for (int mq = 0; mq < MQ; ++mq) {
+    m_i[mq] = NEG_INF;
+    l_i[mq] = 0.0f;
+  }
+
+  // transposing V read: 16-lane block tb, lane ti in the block
+  const int tb = lane >> 4, ti = lane & 15;
+  const int v_d_off = 16 * (tb & 1) + 4 * (ti & 3);  // + dt * 32
+  const int v_k_off = (tb >> 1) * 4 + (ti >> 2);     // + kk * 16 + r * 8
+
+  int slot = 0;
+  for (int j = 0; j < nkv; ++j) {
+    // Tile j has landed for every lane, and every wave is done with the slot
+    // that tile j+1 is about to overwrite.
+    DECA_WAIT_VMCNT(0);
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wave's LDS reads have returned
+    __builtin_amdgcn_s_barrier();
+#if STAGES == 2
+    if (j + 1 < nkv) issue_tile(j + 1, slot ^ 1);
+#endif
+    const unsigned char* k_lds = lds + slot * TILE_BYTES;
+    const unsigned char* v_lds = lds + (STAGES + slot) * TILE_BYTES;
+
+    // ---- S^T = K Q^T ----------------------------------------------------------------
+    floatx16 s_acc[KT][MQ];
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+      for (int mq = 0; mq < MQ; ++mq)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) s_acc[kt][mq][e] = 0.0f;
+#pragma unroll
+    for (int ks = 0; ks < DK; ++ks) {
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt) {
+        const half8 kf = *reinterpret_cast<const half8*>(
+            k_lds + k_chunk_slot(kt * 32 + l32, ks * 2 + half) * 16);
+#pragma unroll
+        for (int mq = 0; mq < MQ; ++mq)
+          s_acc[kt][mq] =
+              __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[mq][ks], s_acc[kt][mq], 0, 0, 0);
+      }
+    }
+
+#if DECA_CAUSAL
+    // Only tiles crossing the diagonal need masking.  Every query sees key 0 in
+    // tile 0, so its running max is finite before a fully masked block shows up.
+    if ((j + 1) * BC - 1 > qt * BR + wave * WQ) {
+#pragma unroll
+      for (int mq = 0; mq < MQ; ++mq) {
+        const int q_idx = qt * BR + wave * WQ + mq * 32 + l32;
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) {
+            const int kv_idx = j * BC + kt * 32 + (e >> 2) * 8 + half * 4 + (e & 3);
+            if (kv_idx > q_idx) s_acc[kt][mq][e] = NEG_INF;
+          }
+      }
+    }
+#endif
+
+    // ---- online softmax: one query column per lane ------------------------------------
+    half8 pf[KK][MQ];
+    float alpha[MQ];
+#pragma unroll
+    for (int mq = 0; mq < MQ; ++mq) {
+      float mx = s_acc[0][mq][0];
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) mx = fmaxf(mx, s_acc[kt][mq][e]);
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float m_new = fmaxf(m_i[mq], mx);
+      alpha[mq] = __builtin_amdgcn_exp2f((m_i[mq] - m_new) * SL2);
+      m_i[mq] = m_new;
+      const float msl = m_new * SL2;
+      float sum = 0.0f;
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const float p = __builtin_amdgcn_exp2f(s_acc[kt][mq][e] * SL2 - msl);
+          s_acc[kt][mq][e] = p;
+          sum += p;
+        }
+#pragma unroll
+        for (int hh = 0; hh < 2; ++hh) {
+          half8 h;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) h[e] = static_cast<_Float16>(s_acc[kt][mq][hh * 8 + e]);
+          pf[kt * 2 + hh][mq] = h;
+        }
+      }
+      l_i[mq] = l_i[mq] * alpha[mq] + sum;
+    }
+    // O^T *= alpha (skipped when no running max moved: multiplying by 1 is exact)
+    {
+      bool moved = false;
+#pragma unroll
+      for (int mq = 0; mq < MQ; ++mq) moved |= (alpha[mq] != 1.0f);
+      if (__builtin_amdgcn_ballot_w64(moved) != 0) {
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+          for (int mq = 0; mq < MQ; ++mq)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) o_acc[dt][mq][e] *= alpha[mq];
+      }
+    }
+
+    // ---- O^T += V^T P^T ----------------------------------------------------------------
+    // k-slot (half, e) of step kk is key row kk*16 + (e/4)*8 + half*4 + e%4: the
+    // order in which the S^T accumulator registers hold the keys.
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        half4 h[2];
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+          const int row = kk * 16 + r * 8 + v_k_off;
+          const int d = dt * 32 + v_d_off;
+          const unsigned char* p = v_lds + v_chunk_slot(row, d >> 3) * 16 + ((d >> 2) & 1) * 8;
+          h[r] = __builtin_bit_cast(half4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4_ptr)(p)));
+        }
+        const half8 vf = __builtin_shufflevector(h[0], h[1], 0, 1, 2, 3, 4, 5, 6, 7);
+#pragma unroll
+        for (int mq = 0; mq < MQ; ++mq)
+          o_acc[dt][mq] =
+              __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf[kk][mq], o_acc[dt][mq], 0, 0, 0);
+      }
+    }
+
+#if STAGES == 2
+    slot ^= 1;
+#else
+    // single slot: everyone must be done reading before the refill
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+    __builtin_amdgcn_s_barrier();
+    if (j + 1 < nkv) issue_tile(j + 1, 0);
+#endif
+  }
+
+  // ---- epilogue: O[q][d] = O^T[d][q] / l ----------------------------------------------
+  // o_acc[dt][mq][e]: q = mq*32 + lane%32, d = dt*32 + (e/4)*8 + half*4 + e%4
+#pragma unroll
+  for (int mq = 0; mq < MQ; ++mq) {
+    const float l = l_i[mq] + __shfl_xor(l_i[mq], 32, 64);
+    const float inv = 1.0f / l;
+    _Float16* o_row = o_base + (mq * 32 + l32) * D_ + half * 4;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        half4 h;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) h[e] = static_cast<_Float16>(o_acc[dt][mq][g * 4 + e] * inv);
+        *reinterpret_cast<half4*>(o_row + dt * 32 + g * 8) = h;
+      }
+  }
+}

@@ -1,0 +1,133 @@
+"""
+FlashAttention-2 style forward kernel: config type, resource estimates,
+validity rules and the specialisation of the HIP template
+`csrc/flash_attn.hip`.
+
+Counterpart of the reference's src/kernels/flash_attn_tir.py.  Layout: Q, K, V,
+O are contiguous [B, H, S, D] float16.
+
+What changes on CDNA4: a wave is 64 lanes and owns a multiple of 32 query rows
+(`Br % (32 * num_warps) == 0` instead of 16, flash_attn_tir.py:72); the two
+products are computed transposed (S^T = K Q^T, O^T = V^T P^T) so that P stays in
+registers between them -- the MFMA accumulator layout is not the operand layout,
+unlike mma.sync m16n8k16 (:8-9); K/V tiles arrive by asynchronous global->LDS
+loads (cp.async, :320-335); Q is read from global memory straight into VGPRs, so
+there is no Q tile in LDS and `q_in_smem` is not offered; the LDS layout is
+always swizzled.
+"""
+
+from __future__ import annotations
+
+import math
+from dataclasses import asdict, dataclass
+
+from deca_amd.kernels.build import (
+    DEFAULT_ARCH, FAST_MATH_OPTIONS, KernelSpec, build_kernel, cached_build, make_spec,
+)
+
+LOG2E = 1.4426950408889634
+NEG_INF = -1e30
+WAVE = 64
+MAX_LDS = 160 * 1024
+TEMPLATE = "flash_attn.hip"
+
+
+@dataclass(frozen=True)
+class FAConfig:
+    Br: int = 128  # Q rows per workgroup
+    Bc: int = 64  # KV rows per pipeline step
+    num_warps: int = 4
+    stages: int = 2  # K/V LDS ring depth
+    q_in_smem: bool = False  # kept for the record format; Q always lives in VGPRs here
+    swizzle: bool = True  # kept for the record format; the LDS layout is always swizzled
+
+    @property
+    def threads(self) -> int:
+        return self.num_warps * WAVE
+
+    def as_dict(self):
+        return asdict(self)
+
+    def __str__(self):
+        return (
+            f"Br={self.Br},Bc={self.Bc},warps={self.num_warps},stages={self.stages},"
+            f"q_smem={int(self.q_in_smem)},swz={int(self.swizzle)}"
+        )
+
+
+def smem_bytes(cfg: FAConfig, D: int) -> int:
+    """`stages` K tiles and `stages` V tiles of Bc x D halves (no Q tile)."""
+    return 2 * cfg.stages * cfg.Bc * D * 2
+
+
+def est_regs_per_thread(cfg: FAConfig, D: int) -> int:
+    """Unified VGPR estimate per lane of the live fragments."""
+    mq = cfg.Br // cfg.num_warps // 32
+    o_acc = (D // 32) * mq * 16
+    s_acc = (cfg.Bc // 32) * mq * 16
+    p_h = s_acc // 2
+    q_frag = mq * (D // 16) * 4
+    kv_frag = 2 * 4 * 2  # a few K / V fragments in flight
+    return o_acc + s_acc + p_h + q_frag + kv_frag + 4 * mq + 40
+
+
+def check_config(cfg: FAConfig, S_q: int, S_kv: int, D: int) -> None:
+    assert D % 64 == 0, "head dim must be a multiple of 64"
+    assert cfg.Br % (32 * cfg.num_warps) == 0
+    assert cfg.Bc % 32 == 0
+    assert S_q % cfg.Br == 0 and S_kv % cfg.Bc == 0
+    cpr = D // 8
+    assert (cfg.Bc * cpr) % cfg.threads == 0
+    assert 2 * (cfg.Bc * cpr) // cfg.threads <= 63
+    assert cfg.threads <= 1024
+    assert cfg.stages in (1, 2)
+    assert not cfg.q_in_smem and cfg.swizzle
+    assert smem_bytes(cfg, D) <= MAX_LDS
+    assert est_regs_per_thread(cfg, D) <= 512
+
+
+def make_flash_attn_fwd(
+    B: int, H: int, S_q: int, S_kv: int, D: int, cfg: FAConfig,
+    softmax_scale: float | None = None, causal: bool = False,
+) -> KernelSpec:
+    """`causal` applies the top-left aligned mask (key j visible to query i iff j <= i).
+    Grid (S_q / Br, B * H), block `threads` (reference: flash_attn_tir.py:147)."""
+    check_config(cfg, S_q, S_kv, D)
+    assert not causal or S_q == S_kv, "causal attention requires S_q == S_kv"
+    scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(D)
+    defines = {
+        "DECA_B": B, "DECA_H": H, "DECA_SQ": S_q, "DECA_SKV": S_kv, "DECA_D": D,
+        "DECA_BR": cfg.Br, "DECA_BC": cfg.Bc, "DECA_NW": cfg.num_warps,
+        "DECA_STAGES": cfg.stages, "DECA_CAUSAL": int(causal),
+        "DECA_SCALE": repr(float(scale)),
+    }
+    return make_spec(
+        TEMPLATE, defines, grid=(S_q // cfg.Br, B * H, 1), block=(cfg.threads, 1, 1), nargs=4,
+        options=FAST_MATH_OPTIONS, meta={"cfg": str(cfg), "causal": causal},
+    )
+
+
+FA_HIPCC_OPTIONS = FAST_MATH_OPTIONS
+
+
+def build_flash_attn_to_file(
+    shape, cfg: FAConfig, softmax_scale, arch: str, path: str, causal: bool = False
+) -> str:
+    """Builds in a worker process (no GPU context needed) and writes a code object."""
+    B, H, S_q, S_kv, D = shape
+    return build_kernel(make_flash_attn_fwd(B, H, S_q, S_kv, D, cfg, softmax_scale, causal), arch, path)
+
+
+def build_flash_attn(spec: KernelSpec, target: str | None = None, dump_dir: str | None = None):
+    """Compiles (or takes from the in-tree cache) and loads the kernel;
+    `dump_dir` keeps the generated ISA for inspection."""
+    import os
+
+    from deca_amd.driver.driver import load_kernel
+
+    arch = target or DEFAULT_ARCH
+    if dump_dir:
+        path = build_kernel(spec, arch, os.path.join(dump_dir, f"fa_{spec.key()}.hsaco"), dump_dir)
+    else:
+        path = cached_build(spec, arch)
+    return load_kernel(spec, path)

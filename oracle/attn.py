@@ -1,0 +1,102 @@
+"""
+numpy restatement of the reference's FlashAttention forward arithmetic.  Test
+infrastructure: see the package docstring for who may import this.
+
+Follows src/kernels/flash_attn_tir.py:
+  layout            :11, :139-142   Q, K, V, O contiguous [B, H, S, D] fp16
+  causal mask       :93, :379-400   key j visible to query i iff j <= i; the
+                                    masked score is -1e30
+  online softmax    :403-438        per KV tile of Bc rows: m' = max(m, rowmax S);
+                                    alpha = exp2((m - m') * sl2);
+                                    p = exp2(S * sl2 - m' * sl2), sl2 = scale * log2e;
+                                    l = l * alpha + sum p (fp32 p); P = fp16(p)
+  second product    :441            O = O * alpha + P V  (fp16 P, fp32 accumulate)
+  normalisation     :444-458        O / l rounded to fp16
+  flop count        src/kernels/attn_bench.py:30-32
+
+`attention_f32` is the plain fp32 softmax(scale * Q K^T + mask) V (the accuracy
+reference); `flash_blockwise` follows the tiled recurrence above, including
+the fp16 rounding of P.
+
+Pinned by (tests/test_oracle_attn.py): torch's softmax-matmul composite on the
+CPU, constant V -> O equals that constant, K = 0 -> uniform attention (O = mean
+of V; causal: prefix mean, which pins the mask direction), the first causal row
+attends to key 0 only, single-tile == multi-tile (pins the online rescale),
+S_q != S_kv, and blockwise == plain within the fp16 rounding of P.
+"""
+
+from __future__ import annotations
+
+import math
+
+import numpy as np
+
+LOG2E = 1.4426950408889634
+NEG_INF = np.float32(-1e30)
+
+
+def default_scale(D: int) -> float:
+    return 1.0 / math.sqrt(D)
+
+
+def attention_f32(q, k, v, scale=None, causal=False) -> np.ndarray:
+    """[B, H, S_q, D] fp32 result (not rounded)."""
+    q = np.asarray(q, np.float32)
+    k = np.asarray(k, np.float32)
+    v = np.asarray(v, np.float32)
+    B, H, S_q, D = q.shape
+    S_kv = k.shape[2]
+    scale = default_scale(D) if scale is None else scale
+    out = np.empty((B, H, S_q, D), np.float32)
+    mask = None
+    if causal:
+        mask = np.arange(S_kv)[None, :] > np.arange(S_q)[:, None]
+    for b in range(B):
+        for h in range(H):
+            s = (q[b, h] @ k[b, h].T) * np.float32(scale)
+            if mask is not None:
+                s = np.where(mask, -np.inf, s)
+            s = s - s.max(axis=-1, keepdims=True)
+            p = np.exp(s, dtype=np.float32)
+            out[b, h] = (p @ v[b, h]) / p.sum(axis=-1, keepdims=True, dtype=np.float32)
+    return out
+
+
+def flash_blockwise(q, k, v, scale=None, causal=False, Br=128, Bc=64) -> np.ndarray:
+    """The tiled online-softmax recurrence; returns fp32 values rounded to fp16."""
+    q = np.asarray(q, np.float32)
+    k = np.asarray(k, np.float32)
+    v = np.asarray(v, np.float32)
+    B, H, S_q, D = q.shape
+    S_kv = k.shape[2]
+    scale = default_scale(D) if scale is None else scale
+    sl2 = np.float32(scale * LOG2E)
+    out = np.empty((B, H, S_q, D), np.float32)
+    for b in range(B):
+        for h in range(H):
+            for q0 in range(0, S_q, Br):
+                qt = q[b, h, q0:q0 + Br]
+                rows = np.arange(q0, q0 + qt.shape[0])
+                m = np.full(qt.shape[0], NEG_INF, np.float32)
+                l = np.zeros(qt.shape[0], np.float32)
+                o = np.zeros((qt.shape[0], D), np.float32)
+                kv_end = min(S_kv, -(-(q0 + Br) // Bc) * Bc) if causal else S_kv
+                for k0 in range(0, kv_end, Bc):
+                    s = qt @ k[b, h, k0:k0 + Bc].T
+                    if causal:
+                        cols = np.arange(k0, k0 + s.shape[1])
+                        s = np.where(cols[None, :] > rows[:, None], NEG_INF, s)
+                    m_new = np.maximum(m, s.max(axis=-1))
+                    alpha = np.exp2((m - m_new) * sl2, dtype=np.float32)
+                    p = np.exp2(s * sl2 - (m_new * sl2)[:, None], dtype=np.float32)
+                    l = l * alpha + p.sum(axis=-1, dtype=np.float32)
+                    p16 = p.astype(np.float16).astype(np.float32)
+                    o = o * alpha[:, None] + p16 @ v[b, h, k0:k0 + Bc]
+                    m = m_new
+                out[b, h, q0:q0 + Br] = o / l[:, None]
+    return out.astype(np.float16).astype(np.float32)
+
+
+def attn_flops(B, H, S_q, S_kv, D, causal=False) -> float:
+    f = 4.0 * B * H * S_q * S_kv * D
+    return f / 2 if causal else f

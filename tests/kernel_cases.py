@@ -1,6 +1,7 @@
 """Kernel specialisations the GPU tests use, listed in one place so that the
 build step can compile all of them ahead of the GPU run."""
 
+from deca_amd.kernels.flash_attn_hip import FAConfig, make_flash_attn_fwd
 from deca_amd.kernels.gemm_hip import GemmConfig, make_gemm_tc
 from deca_amd.kernels.rowwise_hip import RowConfig, make_rowwise
 
@@ -86,5 +87,34 @@ def gemm_specs():
     return [make_gemm_tc(M, N, K, cfg) for M, N, K, cfg in GEMM_CASES + GEMM_FULL]
 
 
+# (B, H, S_q, S_kv, D, causal, cfg): sizes the CPU checker finishes in seconds
+FA_CASES = [
+    (1, 2, 256, 256, 128, False, FAConfig(128, 64, 4, 2)),
+    (1, 2, 256, 256, 128, True, FAConfig(128, 64, 4, 2)),
+    (2, 2, 512, 512, 64, False, FAConfig(128, 64, 4, 2)),
+    (2, 2, 512, 512, 64, True, FAConfig(128, 64, 4, 2)),
+    (1, 2, 512, 512, 128, True, FAConfig(256, 64, 8, 2)),
+    (1, 2, 512, 512, 128, False, FAConfig(256, 32, 8, 1)),
+    (1, 1, 256, 256, 128, True, FAConfig(128, 128, 4, 1)),
+    (1, 2, 256, 256, 64, True, FAConfig(256, 128, 4, 2)),
+    (1, 2, 256, 256, 128, False, FAConfig(128, 32, 2, 2)),
+    (1, 3, 128, 640, 128, False, FAConfig(64, 64, 2, 2)),   # S_q != S_kv
+    (1, 1, 384, 128, 64, False, FAConfig(128, 128, 4, 1)),
+    (1, 1, 128, 128, 128, True, FAConfig(32, 32, 1, 2)),
+]
+
+FA_FULL = [
+    (4, 16, 4096, 4096, 128, False, FAConfig(128, 64, 4, 2)),
+    (4, 16, 4096, 4096, 128, True, FAConfig(128, 64, 4, 2)),
+    (4, 16, 4096, 4096, 64, False, FAConfig(128, 64, 4, 2)),
+    (4, 16, 4096, 4096, 64, True, FAConfig(128, 64, 4, 2)),
+]
+
+
+def fa_specs():
+    return [make_flash_attn_fwd(B, H, Sq, Skv, D, cfg, None, causal)
+            for B, H, Sq, Skv, D, causal, cfg in FA_CASES + FA_FULL]
+
+
 def all_specs():
-    return rowwise_specs() + gemm_specs()
+    return rowwise_specs() + gemm_specs() + fa_specs()

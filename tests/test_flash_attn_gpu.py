@@ -1,0 +1,105 @@
+"""GPU parity of the FlashAttention forward kernel against oracle/attn.py.
+
+Inputs come from a seeded CPU generator and are copied to the device; every
+launch goes through the C ABI.  Accuracy gate (the task's): max|o - ref| <= 2e-3
+against fp32 softmax(scale * Q K^T + mask) V.  The kernel must also sit within
+the same bound of the checker's tiled recurrence (same fp16 rounding of P).
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from kernel_cases import FA_CASES, FA_FULL
+from oracle import attn as oa
+
+pytestmark = pytest.mark.gpu
+
+GATE = 2e-3
+
+
+def _run(B, H, Sq, Skv, D, causal, cfg, q, k, v, scale=None):
+    from deca_amd.kernels.flash_attn_hip import build_flash_attn, make_flash_attn_fwd
+
+    kern = build_flash_attn(make_flash_attn_fwd(B, H, Sq, Skv, D, cfg, scale, causal))
+    o = torch.full((B, H, Sq, D), float("nan"), dtype=torch.float16, device="cuda")
+    kern(q.cuda(), k.cuda(), v.cuda(), o)
+    torch.cuda.synchronize()
+    return o.cpu()
+
+
+def _f32(t):
+    return t.float().numpy()
+
+
+@pytest.mark.parametrize("B,H,Sq,Skv,D,causal,cfg", FA_CASES, ids=lambda v: str(v))
+def test_flash_attn_parity(B, H, Sq, Skv, D, causal, cfg):
+    from deca_amd.kernels.attn_bench import make_qkv_cpu
+
+    print(f"case fa B{B} H{H} Sq{Sq} Skv{Skv} D{D} causal={causal} {cfg}", flush=True)
+    q, k, v = make_qkv_cpu(B, H, Sq, Skv, D, seed=Sq + D)
+    got = _f32(_run(B, H, Sq, Skv, D, causal, cfg, q, k, v))
+    assert np.isfinite(got).all()
+    ref = oa.attention_f32(_f32(q), _f32(k), _f32(v), None, causal)
+    assert np.abs(got - ref).max() <= GATE
+    tiled = oa.flash_blockwise(_f32(q), _f32(k), _f32(v), None, causal, cfg.Br, cfg.Bc)
+    assert np.abs(got - tiled).max() <= GATE
+
+
+def test_flash_attn_closed_forms():
+    """Constant V, zero K (uniform / prefix-mean attention), explicit scale."""
+    from deca_amd.kernels.attn_bench import make_qkv_cpu
+
+    B, H, Sq, Skv, D, _, cfg = FA_CASES[0]
+    q, k, v = make_qkv_cpu(B, H, Sq, Skv, D, seed=7)
+    vc = torch.full_like(v, 0.375)
+    assert (_run(B, H, Sq, Skv, D, False, cfg, q, k, vc).float() - 0.375).abs().max() <= 1e-3
+    k0 = torch.zeros_like(k)
+    got = _f32(_run(B, H, Sq, Skv, D, False, cfg, q, k0, v))
+    assert np.abs(got - _f32(v).mean(axis=2, keepdims=True)).max() <= GATE
+    # causal with K = 0: row i is the mean of V[0..i] -- pins the mask direction
+    got = _f32(_run(B, H, Sq, Skv, D, True, cfg, q, k0, v))
+    prefix = np.cumsum(_f32(v), axis=2) / np.arange(1, Skv + 1)[None, None, :, None]
+    assert np.abs(got - prefix).max() <= GATE
+    # first causal row attends to key 0 only
+    got = _run(B, H, Sq, Skv, D, True, cfg, q, k, v)
+    assert torch.equal(got[:, :, 0], v[:, :, 0])
+    # non-default scale
+    got = _f32(_run(B, H, Sq, Skv, D, False, cfg, q, k, v, scale=0.02))
+    assert np.abs(got - oa.attention_f32(_f32(q), _f32(k), _f32(v), 0.02, False)).max() <= GATE
+
+
+def test_flash_attn_large_scores():
+    """Scores far from zero (|s| ~ 60) must not overflow the exponentials."""
+    from deca_amd.kernels.attn_bench import make_qkv_cpu
+
+    B, H, Sq, Skv, D, _, cfg = FA_CASES[0]
+    q, k, v = make_qkv_cpu(B, H, Sq, Skv, D, seed=9)
+    q = (q.float() * 6).half()
+    k = (k.float() * 6).half()
+    got = _f32(_run(B, H, Sq, Skv, D, False, cfg, q, k, v))
+    assert np.isfinite(got).all()
+    assert np.abs(got - oa.attention_f32(_f32(q), _f32(k), _f32(v), None, False)).max() <= 4e-3
+
+
+@pytest.mark.parametrize("B,H,Sq,Skv,D,causal,cfg", FA_FULL, ids=lambda v: str(v))
+def test_flash_attn_full_size(B, H, Sq, Skv, D, causal, cfg):
+    """Benchmark shapes: a few (batch, head) slices against the CPU checker,
+    every slice against fp32 attention computed on the device."""
+    from deca_amd.kernels.attn_bench import make_qkv_cpu, math_attention
+    from deca_amd.kernels.flash_attn_hip import build_flash_attn, make_flash_attn_fwd
+
+    print(f"full-size fa B{B} H{H} S{Sq} D{D} causal={causal} {cfg}", flush=True)
+    q, k, v = make_qkv_cpu(B, H, Sq, Skv, D, seed=0)
+    kern = build_flash_attn(make_flash_attn_fwd(B, H, Sq, Skv, D, cfg, None, causal))
+    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    o = torch.full((B, H, Sq, D), float("nan"), dtype=torch.float16, device="cuda")
+    kern(qd, kd, vd, o)
+    torch.cuda.synchronize()
+    assert torch.isfinite(o).all()
+    ref = math_attention(qd, kd, vd, causal)
+    assert (o.float() - ref).abs().max().item() <= GATE
+    for b, h in ((0, 0), (B - 1, H - 1)):
+        want = oa.attention_f32(_f32(q[b:b + 1, h:h + 1]), _f32(k[b:b + 1, h:h + 1]),
+                                _f32(v[b:b + 1, h:h + 1]), None, causal)
+        assert np.abs(_f32(o[b:b + 1, h:h + 1].cpu()) - want).max() <= GATE

@@ -1,0 +1,66 @@
+"""Pins the attention checker (oracle/attn.py) without the GPU."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import attn as oa
+
+
+def _qkv(B, H, Sq, Skv, D, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    mk = lambda S: torch.randn(B, H, S, D, generator=g).half().float().numpy()  # noqa: E731
+    return mk(Sq), mk(Skv), mk(Skv)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_plain_matches_torch_composite(causal):
+    q, k, v = _qkv(1, 2, 96, 96, 64)
+    s = torch.from_numpy(q) @ torch.from_numpy(k).transpose(-1, -2) / 8.0
+    if causal:
+        s = s.masked_fill(~torch.ones(96, 96, dtype=torch.bool).tril(), float("-inf"))
+    ref = (torch.softmax(s, -1) @ torch.from_numpy(v)).numpy()
+    assert np.abs(oa.attention_f32(q, k, v, None, causal) - ref).max() < 2e-6
+
+
+def test_constant_v_and_zero_k():
+    q, k, v = _qkv(1, 1, 64, 128, 64, seed=1)
+    vc = np.full_like(v, 0.375)
+    for fn in (oa.attention_f32, lambda *a: oa.flash_blockwise(*a, Br=32, Bc=32)):
+        assert np.abs(fn(q, k, vc, None, False) - 0.375).max() < 1e-3
+    # K = 0: uniform attention -> O is the mean of V; causal: the prefix mean
+    k0 = np.zeros_like(k[:, :, :64])
+    v64 = v[:, :, :64]
+    want = v64.mean(axis=2, keepdims=True)
+    assert np.abs(oa.attention_f32(q, k0, v64, None, False) - want).max() < 1e-5
+    prefix = np.cumsum(v64, axis=2) / np.arange(1, 65)[None, None, :, None]
+    assert np.abs(oa.attention_f32(q, k0, v64, None, True) - prefix).max() < 1e-5
+    got = oa.flash_blockwise(q, k0, v64, None, True, Br=32, Bc=16)
+    assert np.abs(got - prefix).max() < 2e-3
+    # the first causal row sees key 0 only
+    assert np.abs(oa.attention_f32(q, k[:, :, :64], v64, None, True)[0, 0, 0] - v64[0, 0, 0]).max() < 1e-6
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_blockwise_matches_plain_and_tiling_does_not_matter(causal):
+    q, k, v = _qkv(1, 2, 128, 128, 64, seed=2)
+    ref = oa.attention_f32(q, k, v, None, causal)
+    one = oa.flash_blockwise(q, k, v, None, causal, Br=128, Bc=128)
+    many = oa.flash_blockwise(q, k, v, None, causal, Br=32, Bc=32)
+    assert np.abs(one - ref).max() < 2e-3
+    assert np.abs(many - ref).max() < 2e-3
+    assert np.abs(one - many).max() < 2e-3
+
+
+def test_cross_attention_lengths_and_scale():
+    q, k, v = _qkv(2, 1, 64, 192, 128, seed=3)
+    ref = oa.attention_f32(q, k, v, 0.05, False)
+    got = oa.flash_blockwise(q, k, v, 0.05, False, Br=64, Bc=64)
+    assert ref.shape == (2, 1, 64, 128) and np.abs(got - ref).max() < 2e-3
+    # scale matters: a different scale gives a different answer
+    assert np.abs(oa.attention_f32(q, k, v, 0.5, False) - ref).max() > 1e-2
+
+
+def test_flops():
+    assert oa.attn_flops(4, 16, 4096, 4096, 128) == 4.0 * 4 * 16 * 4096 * 4096 * 128
+    assert oa.attn_flops(4, 16, 4096, 4096, 128, True) == 2.0 * 4 * 16 * 4096 * 4096 * 128
