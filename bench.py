@@ -39,7 +39,19 @@ def _row_cfg(d):
     return RowConfig(**d)
 
 
-# name -> description of the workload
+def _gemm_cfg(d):
+    from deca_amd.kernels.gemm_hip import GemmConfig
+
+    return GemmConfig(**d)
+
+
+def _fa_cfg(d):
+    from deca_amd.kernels.flash_attn_hip import FAConfig
+
+    return FAConfig(**d)
+
+
+# name -> description of the workload (the benchmark configurations)
 def workloads():
     t = _tuned()
     w = {}
@@ -50,6 +62,16 @@ def workloads():
     }.items():
         w[name] = {"kind": "rowwise", "op": op, "M": M, "N": N, "dtype": dtype,
                    "cfg": _row_cfg(t[name])}
+    for n in (2048, 4096, 8192, 12288, 16384):
+        name = f"gemm_fp16_{n}"
+        w[name] = {"kind": "gemm", "M": n, "N": n, "K": n, "cfg": _gemm_cfg(t[name])}
+    for D in (128, 64):
+        for causal in (False, True):
+            name = f"fa_fp16_b4h16s4096d{D}" + ("_causal" if causal else "")
+            w[name] = {"kind": "fa", "B": 4, "H": 16, "S": 4096, "D": D, "causal": causal,
+                       "cfg": _fa_cfg(t[name])}
+    for k, v in w.items():
+        v["name"] = k
     return w
 
 
@@ -57,10 +79,19 @@ DEFAULT_WORKLOAD = "rmsnorm_bf16_16384x4096"
 
 
 def _spec(wl):
-    from deca_amd.kernels.rowwise_hip import make_rowwise
-
     if wl["kind"] == "rowwise":
+        from deca_amd.kernels.rowwise_hip import make_rowwise
+
         return make_rowwise(wl["op"], wl["M"], wl["N"], wl["dtype"], wl["cfg"], 1e-6)
+    if wl["kind"] == "gemm":
+        from deca_amd.kernels.gemm_hip import make_gemm_tc
+
+        return make_gemm_tc(wl["M"], wl["N"], wl["K"], wl["cfg"])
+    if wl["kind"] == "fa":
+        from deca_amd.kernels.flash_attn_hip import make_flash_attn_fwd
+
+        return make_flash_attn_fwd(wl["B"], wl["H"], wl["S"], wl["S"], wl["D"], wl["cfg"], None,
+                                   wl["causal"])
     raise ValueError(wl["kind"])
 
 
@@ -77,7 +108,11 @@ def cpu_baseline(wl):
 
     from oracle import baseline as ob
 
-    return ob.time_cpu(wl, torch.get_num_threads())
+    t0 = time.perf_counter()
+    res = ob.time_cpu(wl, torch.get_num_threads())
+    print(f"[bench]   cpu baseline of {wl['name']}: {res['value']:.3g} {res['unit']} on "
+          f"{res['cores']} threads in {time.perf_counter() - t0:.1f} s", file=sys.stderr, flush=True)
+    return res
 
 
 # ---------------------------------------------------------------------------
@@ -133,10 +168,88 @@ def run_rowwise(wl, steps, warmup, with_cpu):
     return res
 
 
+def _timed_steps(kern, sets, steps, warmup):
+    """(wall seconds per step, event seconds per launch) over `steps` launches
+    cycling through the argument sets."""
+    import torch
+
+    n = len(sets)
+    for i in range(warmup):
+        kern(*sets[i % n])
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        kern(*sets[i % n])
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) / steps
+    return wall, kern.time(sets, steps)
+
+
+def run_gemm(wl, steps, warmup, with_cpu):
+    import torch
+
+    from deca_amd.kernels.gemm_bench import gemm_flops, make_inputs
+    from deca_amd.kernels.gemm_hip import build_gemm_tc
+
+    M, N, K = wl["M"], wl["N"], wl["K"]
+    kern = build_gemm_tc(_spec(wl))
+    a, b = make_inputs(M, N, K, seed=0, dist="uniform")
+    c = torch.empty(M, N, dtype=torch.float16, device="cuda")
+    wall, t_k = _timed_steps(kern, [(a, b, c)], steps, warmup)
+    flops = gemm_flops(M, N, K)
+    res = {
+        "workload": wl["name"],
+        "metric": f"fp16 GEMM {M}x{N}x{K} (fp32 accumulate) TFLOPS",
+        "value": flops / wall / 1e12, "unit": "TFLOP/s", "ms_per_step": wall * 1e3,
+        "dtype": "f16 in/out, f32 accumulate", "config": str(wl["cfg"]),
+        "roofline": {"bound": "mfma", "achieved": flops / t_k / 1e12, "peak": MFMA_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": flops / t_k / 1e12 / MFMA_PEAK_TFLOPS,
+                     "traffic": None, "kernel_us": t_k * 1e6, "algorithmic_flops": flops},
+    }
+    if with_cpu:
+        res["cpu_baseline"] = cpu_baseline(wl)
+    del a, b, c
+    torch.cuda.empty_cache()
+    return res
+
+
+def run_fa(wl, steps, warmup, with_cpu):
+    import torch
+
+    from deca_amd.kernels.attn_bench import attn_flops, make_qkv
+    from deca_amd.kernels.flash_attn_hip import build_flash_attn
+
+    B, H, S, D, causal = wl["B"], wl["H"], wl["S"], wl["D"], wl["causal"]
+    kern = build_flash_attn(_spec(wl))
+    q, k, v = make_qkv(B, H, S, S, D, seed=0)
+    o = torch.empty_like(q)
+    wall, t_k = _timed_steps(kern, [(q, k, v, o)], steps, warmup)
+    flops = attn_flops(B, H, S, S, D, causal)
+    res = {
+        "workload": wl["name"],
+        "metric": f"FlashAttention fwd fp16 B{B} H{H} S{S} D{D}{' causal' if causal else ''} TFLOPS",
+        "value": flops / wall / 1e12, "unit": "TFLOP/s", "ms_per_step": wall * 1e3,
+        "dtype": "f16 in/out, f32 accumulate", "config": str(wl["cfg"]),
+        "roofline": {"bound": "mfma", "achieved": flops / t_k / 1e12, "peak": MFMA_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": flops / t_k / 1e12 / MFMA_PEAK_TFLOPS,
+                     "traffic": None, "kernel_us": t_k * 1e6, "algorithmic_flops": flops},
+    }
+    if with_cpu:
+        res["cpu_baseline"] = cpu_baseline(wl)
+    del q, k, v, o
+    torch.cuda.empty_cache()
+    return res
+
+
 def run(wl, steps, warmup, with_cpu=True):
-    if wl["kind"] == "rowwise":
-        return run_rowwise(wl, steps, warmup, with_cpu)
-    raise ValueError(wl["kind"])
+    t0 = time.perf_counter()
+    print(f"[bench] {wl['name']} ...", file=sys.stderr, flush=True)
+    res = {"rowwise": run_rowwise, "gemm": run_gemm, "fa": run_fa}[wl["kind"]](
+        wl, steps, warmup, with_cpu)
+    print(f"[bench] {wl['name']}: {res['value']:.1f} {res['unit']} "
+          f"({100 * res['roofline']['frac']:.1f}% of peak) in {time.perf_counter() - t0:.1f} s",
+          file=sys.stderr, flush=True)
+    return res
 
 
 def main():
@@ -158,8 +271,6 @@ def main():
         print("bench.py needs a GPU (the kernels have no host path)", file=sys.stderr)
         sys.exit(1)
     wls = workloads()
-    for k, v in wls.items():
-        v["name"] = k
     head = run(wls[args.workload], args.steps, args.warmup, not args.no_cpu)
     out = {
         "metric": head["metric"],
@@ -180,8 +291,11 @@ def main():
     if "cpu_baseline" in head:
         out["cpu_baseline"] = head["cpu_baseline"]
     if not args.no_extra:
+        # the other benchmark configurations, with fewer steps each so that the
+        # default run stays within a few minutes
+        k = max(5, min(args.steps, 30))
         out["results"] = [head] + [
-            run(wl, args.steps, args.warmup, not args.no_cpu)
+            run(wl, k, min(args.warmup, 5), not args.no_cpu)
             for name, wl in wls.items() if name != args.workload
         ]
     print(json.dumps(out))

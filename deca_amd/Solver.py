@@ -32,13 +32,15 @@ class _IntOps:
     def const(v):
         return int(v)
 
+    # Division by zero follows the bit-vector theory (all ones / the dividend),
+    # so that both back ends agree on partially defined expressions.
     @staticmethod
     def udiv(a, b):
-        return a // b
+        return a // b if b else (1 << 32) - 1
 
     @staticmethod
     def urem(a, b):
-        return a % b
+        return a % b if b else a
 
     @staticmethod
     def ule(a, b):
@@ -241,3 +243,171 @@ def solve_rowwise(
         )
         for tpr, rpb, vec, mode, unroll, hint in _enumerate(ROWWISE_DOMAINS, cons, count, backend)
     ]
+
+
+# ---------------------------------------------------------------------------
+# FP16 MFMA GEMM
+# ---------------------------------------------------------------------------
+GEMM_DOMAINS = {
+    "bm": (64, 128, 256),
+    "bn": (64, 128, 256),
+    "bk": (32, 64),
+    "wm": (32, 64, 128),
+    "wn": (32, 64, 128),
+    "st": (1, 2, 3, 4),
+    "epi": (0, 1),
+    "direct": (0, 1),
+}
+GEMM_RASTERS = (1, 2, 4, 8, 16)
+
+
+def _gemm_constraints(arch, M: int, N: int, K: int, type_size: int):
+    from deca_amd.kernels.gemm_hip import EPI_PAD
+
+    wave = arch.warp_size
+    simds = arch.simds_per_cu
+
+    def build(o, v):
+        bm, bn, bk, wm, wn, st, epi, direct = (v[k] for k in GEMM_DOMAINS)
+        c = o.const
+        m_, n_, k_ = c(M), c(N), c(K)
+        waves = o.udiv(bm, wm) * o.udiv(bn, wn)
+        threads = waves * wave
+        out = [
+            # wave tiles divide the workgroup tile, workgroup tiles divide the problem
+            o.eq(o.urem(bm, wm), c(0)), o.eq(o.urem(bn, wn), c(0)),
+            o.eq(o.urem(m_, bm), c(0)), o.eq(o.urem(n_, bn), c(0)), o.eq(o.urem(k_, bk), c(0)),
+            # ring depth: asynchronous direct loads use 2..4 slots, staged loads 1..2,
+            # never more than there are K tiles
+            o.implies(o.eq(direct, c(1)), o.uge(st, c(2))),
+            o.implies(o.eq(direct, c(0)), o.ule(st, c(2))),
+            o.ule(st, o.udiv(k_, bk)),
+            # 1 to 16 waves per workgroup
+            o.uge(threads, c(wave)), o.ule(threads, c(arch.max_threads_per_block)),
+            # cooperative 16-byte loads (and epilogue stores) evenly cover the tiles
+            o.eq(o.urem(bm * o.udiv(bk, c(8)), threads), c(0)),
+            o.eq(o.urem(bk * o.udiv(bn, c(8)), threads), c(0)),
+            o.implies(o.eq(epi, c(1)), o.eq(o.urem(bm * o.udiv(bn, c(8)), threads), c(0))),
+        ]
+        # LDS: `st` A and B tiles; the staged epilogue reuses them
+        pipe = st * (bm * bk + bk * bn) * type_size
+        epi_bytes = o.ite(o.eq(epi, c(1)), bm * (bn + EPI_PAD) * type_size, c(0))
+        out += [o.ule(pipe, c(arch.max_dyn_smem_per_block)),
+                o.ule(epi_bytes, c(arch.max_dyn_smem_per_block))]
+        # unified VGPRs: fp32 accumulators + two fragment sets + staging + bookkeeping,
+        # as in gemm_hip.est_regs_per_thread
+        acc = o.udiv(wm * wn, c(wave))
+        frags = 4 * (o.udiv(wm, c(32)) + o.udiv(wn, c(32)))
+        chunks = o.udiv(o.udiv(bm * bk + bk * bn, c(8)), threads)
+        staging = o.ite(o.eq(direct, c(1)), chunks, chunks * 4)
+        regs = acc + 2 * frags + staging + 40
+        regs8 = o.udiv(regs + 7, c(8)) * 8
+        waves_per_simd = o.udiv(waves + (simds - 1), c(simds))
+        out += [o.ule(regs, c(arch.vgprs_per_simd)),
+                o.ule(regs8 * waves_per_simd, c(arch.vgprs_per_simd))]
+        # enough workgroups to give every CU at least one
+        out.append(o.uge(o.udiv(m_, bm) * o.udiv(n_, bn), c(arch.sm_nums)))
+        return out
+
+    return build
+
+
+def solve_gemm_tc(arch, M: int, N: int, K: int, type_size: int = 2, count: int = 8192,
+                  backend: str = "auto"):
+    """
+    Enumerate FP16 MFMA GEMM tile configurations (see `GemmConfig`).
+    Args:
+        arch: Arch, the target GPU
+        M, N, K: the GEMM shape (C[M, N] = A[M, K] @ B[K, N])
+        type_size: bytes per input element (2 for fp16)
+        count: the maximum number of solutions to find
+    Returns:
+        list of GemmConfig
+    """
+    from deca_amd.kernels.gemm_hip import GemmConfig
+
+    tiles = _enumerate(GEMM_DOMAINS, _gemm_constraints(arch, M, N, K, type_size), count, backend)
+    results = []
+    for bm, bn, bk, wm, wn, st, epi, direct in tiles:
+        # The rasterisation group only needs to divide the workgroup rows and the
+        # XCD remap needs a multiple of 8 workgroups; neither interacts with the
+        # other constraints, so both are expanded here (reference: Solver.py:550-558).
+        xcd = ((M // bm) * (N // bn)) % arch.num_xcd == 0
+        for ras in GEMM_RASTERS:
+            if (M // bm) % ras == 0:
+                results.append(GemmConfig(BM=bm, BN=bn, BK=bk, warp_m=wm, warp_n=wn, stages=st,
+                                          raster=ras, epi_smem=bool(epi), xcd=xcd,
+                                          direct=bool(direct)))
+    return results[:count]
+
+
+# ---------------------------------------------------------------------------
+# FlashAttention forward
+# ---------------------------------------------------------------------------
+FA_DOMAINS = {
+    "br": (32, 64, 128, 256),
+    "bc": (32, 64, 128),
+    "nw": (1, 2, 4, 8),
+    "st": (1, 2),
+}
+
+
+def _fa_constraints(arch, B: int, H: int, S_q: int, S_kv: int, D: int, type_size: int,
+                    max_est_regs: int):
+    wave = arch.warp_size
+    simds = arch.simds_per_cu
+
+    def build(o, v):
+        br, bc, nw, st = (v[k] for k in FA_DOMAINS)
+        c = o.const
+        threads = nw * wave
+        cpr = D // 8
+        out = [
+            # each wave owns a multiple of 32 Q rows; the tiles divide the sequences
+            o.eq(o.urem(br, nw * 32), c(0)),
+            o.eq(o.urem(c(S_q), br), c(0)), o.eq(o.urem(c(S_kv), bc), c(0)),
+            # do not pipeline deeper than the number of KV tiles
+            o.ule(st, o.udiv(c(S_kv), bc)),
+            # cooperative 16-byte loads evenly cover a K/V tile; the outstanding
+            # loads of one tile pair fit the 6-bit vector-memory counter
+            o.eq(o.urem(bc * cpr, threads), c(0)),
+            o.ule(o.udiv(bc * cpr, threads) * 2, c(63)),
+            o.ule(threads, c(arch.max_threads_per_block)),
+            # LDS: `st` K tiles and `st` V tiles
+            o.ule(st * bc * (2 * D * type_size), c(arch.max_dyn_smem_per_block)),
+        ]
+        # registers: O^T accumulator + S^T accumulator + P + Q fragments + K/V fragments
+        mq = o.udiv(br, nw * 32)
+        o_acc = mq * (D // 32 * 16)
+        s_acc = mq * o.udiv(bc, c(2))
+        p_h = mq * o.udiv(bc, c(4))
+        q_frag = mq * (D // 16 * 4)
+        regs = o_acc + s_acc + p_h + q_frag + 16 + mq * 4 + 40
+        regs8 = o.udiv(regs + 7, c(8)) * 8
+        waves_per_simd = o.udiv(nw + (simds - 1), c(simds))
+        out += [o.ule(regs, c(max_est_regs)), o.ule(regs8 * waves_per_simd, c(arch.vgprs_per_simd))]
+        # enough workgroups to give every CU at least one
+        out.append(o.uge(o.udiv(c(S_q), br) * (B * H), c(arch.sm_nums)))
+        return out
+
+    return build
+
+
+def solve_flash_attn(arch, B: int, H: int, S_q: int, S_kv: int, D: int, type_size: int = 2,
+                     max_est_regs: int = 512, count: int = 256, backend: str = "auto"):
+    """
+    Enumerate FlashAttention forward tile configurations.
+    Args:
+        arch: Arch, the target GPU
+        B, H, S_q, S_kv, D: the attention shape
+        type_size: bytes per input element (2 for fp16)
+        max_est_regs: upper bound of the estimated unified VGPRs per lane
+        count: the maximum number of solutions to find
+    Returns:
+        list of FAConfig
+    """
+    from deca_amd.kernels.flash_attn_hip import FAConfig
+
+    cons = _fa_constraints(arch, B, H, S_q, S_kv, D, type_size, max_est_regs)
+    return [FAConfig(Br=br, Bc=bc, num_warps=nw, stages=st)
+            for br, bc, nw, st in _enumerate(FA_DOMAINS, cons, count, backend)]

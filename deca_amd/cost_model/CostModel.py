@@ -96,3 +96,180 @@ def rank_rowwise_configs(configs, arch, op: str, M: int, N: int, top_n: int | No
     """Sort row-wise configs by `rowwise_score` (best first)."""
     ranked = sorted(configs, key=lambda c: rowwise_score(c, arch, op, M, N), reverse=True)
     return ranked[:top_n] if top_n else ranked
+
+
+# ---------------------------------------------------------------------------
+# FP16 MFMA GEMM
+# ---------------------------------------------------------------------------
+def gemm_tc_occupancy(cfg, arch) -> int:
+    """Resident workgroups per CU of an FP16 MFMA GEMM config."""
+    from deca_amd.kernels.gemm_hip import est_regs_per_thread, smem_bytes
+
+    wgs, _ = cu_occupancy(arch, est_regs_per_thread(cfg), smem_bytes(cfg), cfg.threads)
+    return max(int(wgs), 1)
+
+
+def gemm_wave_dram_bytes_per_flop(cfg, arch, M: int, N: int, K: int, slots: int) -> float:
+    """HBM bytes per FLOP of A / B (fp16) for one wave of `slots` concurrent
+    workgroups.  With grouped rasterisation a wave covers `rows` workgroup rows
+    x `cols` columns; every A row block and B column block of the wave is
+    fetched once.  Operands that fit comfortably in the Infinity Cache are
+    fetched once overall (reference: CostModel.py:182-196, with L2 -> MALL)."""
+    cache = getattr(arch, "mall_bytes", arch.l2_bytes)
+    if (M * K + K * N) * 2 <= 0.5 * cache:
+        return (M * K + K * N) * 2 / (2.0 * M * N * K)
+    GM, GN = M // cfg.BM, N // cfg.BN
+    g = cfg.raster
+    cols = min(GN, math.ceil(slots / g))
+    rows = min(GM, g * math.ceil(slots / (g * GN)))
+    tiles = min(slots, GM * GN)
+    return (rows * cfg.BM + cols * cfg.BN) / (tiles * cfg.BM * cfg.BN)
+
+
+def gemm_mma_peak(cfg, arch) -> float:
+    """MFMA peak (GFLOPS) with fp32 accumulation, the only mode of the matrix cores."""
+    return arch.peak_mma_sync_flops
+
+
+def gemm_tc_score(cfg, arch, M: int, N: int, K: int) -> float:
+    """
+    Heuristic score of an FP16 MFMA GEMM config.
+
+    Per-CU time per FLOP of the main loop, as a roofline whose non-bottleneck
+    terms only partially overlap:
+    - matrix cores (MFMA 32x32x16, fp32 accumulation)
+    - LDS: every wave reads (WM + WN) * 16 * 2 bytes per k16 step for
+      2 * WM * WN * 16 FLOPs, and the workgroup fills (BM + BN) * BK * 2 bytes
+      per stage (through the LDS write port unless the loads are direct)
+    - L2: every workgroup streams its A rows and B columns,
+      (BM + BN) / (BM * BN) B/FLOP, from the L2 of its XCD; without the XCD remap
+      neighbouring tiles land on different XCDs and share nothing there
+    - HBM / Infinity Cache: the unique A / B blocks of one wave of workgroups
+    Then:
+    - wave efficiency of the workgroup grid
+    - issue: with one wave per SIMD nothing covers that wave's own waits (LDS
+      latency before the first MFMA of a k-step, the barrier); a second wave does
+    - pipelining: bytes in flight ((stages - 1) tiles per workgroup, or one tile
+      for the VGPR-staged ring) vs. Little's law on the L2 stream; excess
+      stages are penalised by `arch.gemm_excess_stage_penalty`
+    - one barrier per BK stage
+    - epilogue: C is written once; direct stores are 8-byte row segments, the
+      staged epilogue writes 16-byte coalesced chunks
+    """
+    wgs = gemm_tc_occupancy(cfg, arch)
+    slots = arch.sm_nums * wgs
+    grid = (M // cfg.BM) * (N // cfg.BN)
+    wave_eff = _wave_efficiency(grid, slots)
+    waves_per_simd = wgs * cfg.num_warps / arch.simds_per_cu
+    hiding = min(1.0, 0.82 + 0.09 * min(waves_per_simd, 2.0)) if waves_per_simd >= 1 else \
+        0.82 * waves_per_simd
+
+    cus = arch.sm_nums
+    wm, wn = cfg.warp_m, cfg.warp_n
+    peak = gemm_mma_peak(cfg, arch)
+    t_mma = cus / (peak * 1e9)
+    fill_bpf = (cfg.BM + cfg.BN) / (cfg.BM * cfg.BN)
+    lds_bpf = (wm + wn) / (wm * wn) + (0.0 if cfg.direct else fill_bpf)
+    t_lds = lds_bpf / arch.smem_bw_per_sm
+    l2_bpf = fill_bpf * (1.0 if cfg.xcd else 1.5)
+    t_l2 = l2_bpf * cus / (arch.l2_bw * 1e9)
+    dram_bpf = gemm_wave_dram_bytes_per_flop(cfg, arch, M, N, K, slots)
+    t_dram = dram_bpf * cus / (arch.dram_bw * 1e9)
+    terms = sorted([t_mma, t_lds, t_l2, t_dram])
+    t_flop = terms[-1] + 0.25 * sum(terms[:-1])
+
+    # Bytes per CU that must be in flight to cover ~1.5 us of L2 / fabric latency.
+    need = fill_bpf / t_mma * 1.5e-6
+    stage_bytes = wgs * (cfg.BM + cfg.BN) * cfg.BK * 2
+    depth = (cfg.stages - 1) if cfg.direct else 1
+    in_flight = max(depth, 0.5) * stage_bytes
+    pipe = min(1.0, in_flight / need) ** 0.5
+    excess = max(0, depth - math.ceil(need / stage_bytes))
+    pipe *= 1.0 - getattr(arch, "gemm_excess_stage_penalty", 0.0) * excess
+
+    # CU cycles per stage at the MFMA rate vs. ~200 cycles of barrier + refill issue
+    flops_per_cycle = peak * 1e9 / cus / arch.sm_clock_hz
+    stage_cycles = 2 * cfg.BM * cfg.BN * cfg.BK / flops_per_cycle
+    sync_eff = 1.0 / (1.0 + 200.0 / wgs / stage_cycles)
+
+    epi_eff = 1.0 if cfg.epi_smem else 0.5
+    t_epi = (1.0 / K) / epi_eff * cus / (arch.dram_bw * 1e9)
+    t_epi *= 1.0 if wgs == 1 else 0.4
+
+    return wave_eff * hiding * pipe * sync_eff / ((t_flop + t_epi) / t_mma)
+
+
+def rank_gemm_configs(configs, arch, M: int, N: int, K: int, top_n: int | None = None):
+    """Sort FP16 MFMA GEMM configs by `gemm_tc_score` (best first)."""
+    ranked = sorted(configs, key=lambda c: gemm_tc_score(c, arch, M, N, K), reverse=True)
+    return ranked[:top_n] if top_n else ranked
+
+
+# ---------------------------------------------------------------------------
+# FlashAttention forward
+# ---------------------------------------------------------------------------
+def fa_occupancy(cfg, arch, D: int, grid: int):
+    """Returns (resident workgroups per CU, share of the wave slots in use)."""
+    from deca_amd.kernels.flash_attn_hip import est_regs_per_thread, smem_bytes
+
+    wgs, _ = cu_occupancy(arch, est_regs_per_thread(cfg, D), smem_bytes(cfg, D), cfg.threads)
+    wgs = max(int(wgs), 1)
+    return wgs, wgs * cfg.num_warps / arch.max_resident_warps_per_sm
+
+
+def fa_score(cfg, arch, shape, causal: bool = False) -> float:
+    """
+    Heuristic score of a FlashAttention config.
+
+    - roofline of one CU per FLOP: matrix-core time vs. LDS time (every wave
+      reads the whole K and V tile for its WQ query rows: 1 / WQ bytes per
+      FLOP) vs. L2 time (every workgroup streams K/V once: 1 / Br bytes per
+      FLOP); the non-bottleneck terms only partially overlap
+    - softmax: per score element one exponential (quarter rate) plus ~4 full
+      rate operations on the vector ALU, which runs beside the matrix cores
+      only when another wave on the SIMD has MFMAs to issue
+    - wave efficiency: the tail of the last wave of workgroups is wasted
+    - barriers: one per KV step, hidden better by several smaller resident
+      workgroups (`arch.fa_cta_sync_penalty`)
+    - a 2-deep K/V ring hides the global->LDS latency; a single slot exposes it
+    - causal: tiles crossing the diagonal are computed in full, so only the
+      useful fraction of the computed score tiles counts
+    """
+    B, H, S_q, S_kv, D = shape
+    grid = (S_q // cfg.Br) * B * H
+    wgs, _ = fa_occupancy(cfg, arch, D, grid)
+    slots = arch.sm_nums * wgs
+    wave_eff = _wave_efficiency(grid, slots)
+
+    waves_per_simd = wgs * cfg.num_warps / arch.simds_per_cu
+    wq = cfg.Br // cfg.num_warps
+    cus = arch.sm_nums
+    t_mma = cus / (arch.peak_mma_sync_flops * 1e9)
+    t_lds = (1.0 / wq) / arch.smem_bw_per_sm
+    t_l2 = (1.0 / cfg.Br) * cus / (arch.l2_bw * 1e9)
+    # vector-ALU time per FLOP: (4 + 4) lane-cycles per score element, 4 * D FLOPs each
+    valu_rate = cus * arch.simds_per_cu * 16 * arch.sm_clock_hz  # lane-ops per second
+    t_valu = (8.0 / (4.0 * D)) * cus / valu_rate
+    overlap = min(1.0, max(0.0, waves_per_simd - 1.0))  # share of VALU work hidden by other waves
+    terms = sorted([t_mma, t_lds, t_l2])
+    t_flop = terms[-1] + 0.3 * (terms[0] + terms[1]) + (1.0 - 0.8 * overlap) * t_valu
+    t_flop = max(t_flop, t_valu)
+
+    pipe = 1.0 if cfg.stages >= 2 else 0.96
+    sync = 1.0 / (1.0 + getattr(arch, "fa_cta_sync_penalty", 0.0) * cfg.num_warps / 4 / wgs)
+    # longer KV steps amortise the per-step max / rescale / barrier
+    step = 1.0 / (1.0 + 0.06 * 64 / cfg.Bc)
+
+    useful = 1.0
+    if causal:
+        nq = S_q // cfg.Br
+        computed = sum(-(-(i + 1) * cfg.Br // cfg.Bc) * cfg.Bc for i in range(nq)) * cfg.Br
+        useful = S_q * (S_q + 1) / 2 / computed
+
+    return wave_eff * pipe * sync * step * useful / (t_flop / t_mma)
+
+
+def rank_fa_configs(configs, arch, shape, causal: bool = False, top_n: int | None = None):
+    """Sort FlashAttention configs by `fa_score` (best first)."""
+    ranked = sorted(configs, key=lambda c: fa_score(c, arch, shape, causal), reverse=True)
+    return ranked[:top_n] if top_n else ranked
