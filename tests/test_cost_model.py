@@ -1,0 +1,100 @@
+"""Host tests of the analytical ranking: occupancy arithmetic checked by hand,
+closed-form pieces, and the monotonic behaviour each term is there for."""
+
+import math
+
+import pytest
+
+from deca_amd.arch import MI355X
+from deca_amd.cost_model import CostModel as cm
+from deca_amd.driver.driver import cu_occupancy
+from deca_amd.kernels.flash_attn_hip import FAConfig
+from deca_amd.kernels.gemm_hip import GemmConfig
+from deca_amd.kernels.rowwise_hip import RowConfig
+
+ARCH = MI355X()
+
+
+def test_cu_occupancy_by_hand():
+    # 256 lanes = 4 waves = one per SIMD; 128 VGPRs -> 4 waves per SIMD -> 4 workgroups
+    assert cu_occupancy(ARCH, 128, 0, 256) == (4, 4)
+    # 64 VGPRs -> 8 waves per SIMD (the cap), 32 waves per CU / 4 per workgroup
+    assert cu_occupancy(ARCH, 64, 0, 256) == (8, 8)
+    # more than 256 VGPRs: one wave per SIMD
+    assert cu_occupancy(ARCH, 300, 0, 256) == (1, 1)
+    # LDS bound: 64 KiB per workgroup -> 2 workgroups in 160 KiB
+    assert cu_occupancy(ARCH, 64, 64 * 1024, 256)[0] == 2
+    # a single-wave workgroup: 4 SIMDs x 5 waves of 100 (-> 104) VGPRs... 512 // 104 = 4
+    assert cu_occupancy(ARCH, 100, 0, 64) == (16, 4)
+    # 512 lanes = 8 waves = 2 per SIMD; 250 (-> 256) VGPRs -> 2 waves per SIMD -> 1 workgroup
+    assert cu_occupancy(ARCH, 250, 0, 512) == (1, 2)
+    assert cu_occupancy(ARCH, 600, 0, 64) == (0, 0)
+
+
+def test_wave_efficiency():
+    assert cm._wave_efficiency(512, 256) == 1.0
+    assert cm._wave_efficiency(257, 256) == pytest.approx(257 / 512)
+
+
+def test_rowwise_score_terms():
+    M, N = 16384, 4096
+    base = RowConfig(128, 1, 8)
+    s0 = cm.rowwise_score(base, ARCH, "softmax", M, N)
+    assert 0 < s0 <= 1
+    # non-temporal hints, 16-byte accesses and reg mode each help
+    assert cm.rowwise_score(RowConfig(128, 1, 8, hint=True), ARCH, "softmax", M, N) > s0
+    assert cm.rowwise_score(RowConfig(128, 1, 4), ARCH, "softmax", M, N) < s0
+    assert cm.rowwise_score(RowConfig(128, 1, 8, "twopass", 2), ARCH, "softmax", M, N) < s0
+    # a ragged tail idles lanes
+    assert cm.rowwise_score(base, ARCH, "softmax", M, 4104) < s0
+    ranked = cm.rank_rowwise_configs([RowConfig(1024, 1, 4), base], ARCH, "softmax", M, N, top_n=1)
+    assert ranked == [base]
+    assert cm.rowwise_occupancy(RowConfig(64, 1, 8), ARCH, "softmax", N) >= 1
+
+
+def test_gemm_dram_bytes_per_flop_closed_form():
+    cfg = GemmConfig(256, 256, 64, 128, 64, 2, 4)
+    # operands that fit half the Infinity Cache are fetched once overall
+    n = 4096
+    assert cm.gemm_wave_dram_bytes_per_flop(cfg, ARCH, n, n, n, 256) == pytest.approx(
+        (2 * n * n * 2) / (2.0 * n**3))
+    # large problem: one wave of 256 tiles in groups of 4 rows covers 4 rows x 64 columns
+    n = 16384
+    got = cm.gemm_wave_dram_bytes_per_flop(cfg, ARCH, n, n, n, 256)
+    assert got == pytest.approx((4 * 256 + 64 * 256) / (256 * 256 * 256))
+
+
+def test_gemm_score_terms():
+    n = 8192
+    good = GemmConfig(256, 256, 64, 128, 64, 2, 4)
+    s = cm.gemm_tc_score(good, ARCH, n, n, n)
+    assert 0 < s <= 1
+    # small tiles need more LDS and L2 bytes per FLOP
+    assert cm.gemm_tc_score(GemmConfig(64, 64, 64, 32, 32, 2, 4), ARCH, n, n, n) < s
+    # a staged ring pays the LDS write traffic that direct loads avoid
+    assert cm.gemm_tc_score(GemmConfig(256, 256, 64, 128, 64, 2, 4, direct=False), ARCH, n, n, n) < s
+    # without the XCD remap the L2 term grows
+    assert cm.gemm_tc_score(GemmConfig(256, 256, 64, 128, 64, 2, 4, xcd=False), ARCH, n, n, n) <= s
+    assert cm.gemm_tc_occupancy(good, ARCH) == 1
+    top = cm.rank_gemm_configs([GemmConfig(64, 64, 64, 32, 32, 2, 4), good], ARCH, n, n, n, top_n=1)
+    assert top == [good]
+    assert cm.gemm_mma_peak(good, ARCH) == ARCH.peak_mma_sync_flops
+
+
+def test_fa_score_terms():
+    shape = (4, 16, 4096, 4096, 128)
+    a = FAConfig(256, 128, 8, 2)
+    s = cm.fa_score(a, ARCH, shape)
+    assert s > 0
+    assert cm.fa_score(FAConfig(256, 128, 8, 1), ARCH, shape) < s       # single slot exposes latency
+    assert cm.fa_score(a, ARCH, shape, causal=True) < s                  # diagonal tiles are wasted work
+    # causal useful fraction: Br = Bc = S means one tile, half of it useful
+    one = FAConfig(256, 128, 8, 1)
+    nq, computed = 4096 // 256, 0
+    for i in range(nq):
+        computed += math.ceil((i + 1) * 256 / 128) * 128 * 256
+    ratio = cm.fa_score(one, ARCH, shape, True) / cm.fa_score(one, ARCH, shape, False)
+    assert ratio == pytest.approx(4096 * 4097 / 2 / computed)
+    wgs, share = cm.fa_occupancy(a, ARCH, 128, 1024)
+    assert wgs == 1 and share == pytest.approx(8 / 32)
+    assert cm.rank_fa_configs([FAConfig(32, 32, 1, 1), a], ARCH, shape, top_n=1) == [a]

@@ -1,0 +1,155 @@
+"""Host tests of the configuration solver: every emitted config is valid for
+its kernel template, the enumeration is exhaustive (cross-checked against an
+independent filter over the raw domain product), and the documented rules
+(reg vs twopass, raster / XCD expansion) hold."""
+
+import itertools
+
+import pytest
+
+from deca_amd import Solver
+from deca_amd.arch import MI355X
+from deca_amd.kernels import flash_attn_hip as fa
+from deca_amd.kernels import gemm_hip as gm
+from deca_amd.kernels import rowwise_hip as rw
+
+ARCH = MI355X()
+
+
+def test_intops_follow_bitvector_division():
+    o = Solver._IntOps
+    assert o.udiv(7, 2) == 3 and o.urem(7, 2) == 1
+    assert o.udiv(7, 0) == 2**32 - 1 and o.urem(7, 0) == 7
+    assert o.implies(False, False) and not o.implies(True, False)
+    assert o.ite(True, 1, 2) == 1 and o.all_of(True, True) and o.any_of(False, True)
+
+
+@pytest.mark.parametrize("op,M,N", [("softmax", 16384, 4096), ("rmsnorm", 16384, 4096),
+                                    ("rmsnorm", 8192, 8192), ("softmax", 4096, 1024),
+                                    ("softmax", 1024, 32000), ("softmax", 8192, 128256)])
+def test_rowwise_configs_are_valid_and_exhaustive(op, M, N):
+    configs = Solver.solve_rowwise(ARCH, op, M, N)
+    assert configs and len(set(configs)) == len(configs)
+    for cfg in configs:
+        rw.check_config(cfg, op, M, N, "float16")
+        assert M // cfg.rows_per_block >= ARCH.sm_nums
+        assert cfg.threads_per_row * cfg.vec <= N
+    # independent enumeration: raw product filtered by the kernel's own rules
+    want = set()
+    for tpr, rpb, vec, mode, unroll, hint in itertools.product(
+            (16, 32, 64, 128, 256, 512, 1024), (1, 2, 4, 8, 16), (4, 8), ("reg", "twopass"),
+            (1, 2, 4), (False, True)):
+        cfg = rw.RowConfig(tpr, rpb, vec, mode, unroll, hint)
+        try:
+            rw.check_config(cfg, op, M, N, "float16")
+        except AssertionError:
+            continue
+        if M // rpb < ARCH.sm_nums or tpr * vec > N:
+            continue
+        if mode == "reg" and (unroll != 1 or rw.num_chunks(cfg, N) > 32):
+            continue
+        if rw.est_regs_per_thread(cfg, N, op) > ARCH.max_arch_vgprs:
+            continue
+        want.add(cfg)
+    has_reg = any(c.mode == "reg" for c in want)
+    if N < 16384 and has_reg:
+        want = {c for c in want if c.mode == "reg"}
+    assert set(configs) == want
+
+
+def test_rowwise_mode_rules():
+    assert all(c.mode == "reg" for c in Solver.solve_rowwise(ARCH, "softmax", 16384, 4096))
+    modes = {c.mode for c in Solver.solve_rowwise(ARCH, "softmax", 1024, 32000)}
+    assert modes == {"reg", "twopass"}  # N >= 16384: both offered
+    # a row too long for the register file: only twopass survives
+    long_row = Solver.solve_rowwise(ARCH, "softmax", 1024, 1 << 19)
+    assert long_row and {c.mode for c in long_row} == {"twopass"}
+    # lowering the threshold admits twopass for short rows too
+    both = Solver.solve_rowwise(ARCH, "softmax", 16384, 4096, twopass_min_n=1024)
+    assert {c.mode for c in both} == {"reg", "twopass"}
+    assert len(Solver.solve_rowwise(ARCH, "softmax", 16384, 4096, count=5)) == 5
+    assert Solver.solve_rowwise(ARCH, "softmax", 64, 4096) == []  # fewer rows than CUs
+
+
+@pytest.mark.parametrize("n", [2048, 4096, 8192])
+def test_gemm_configs_are_valid(n):
+    configs = Solver.solve_gemm_tc(ARCH, n, n, n)
+    assert configs and len(set(configs)) == len(configs)
+    for cfg in configs:
+        gm.check_config(cfg, n, n, n)
+        assert (n // cfg.BM) * (n // cfg.BN) >= ARCH.sm_nums
+        assert (n // cfg.BM) % cfg.raster == 0
+        assert cfg.xcd == (((n // cfg.BM) * (n // cfg.BN)) % 8 == 0)
+        assert cfg.stages >= 2 if cfg.direct else cfg.stages <= 2
+    if n >= 4096:
+        assert gm.GemmConfig(256, 256, 64, 128, 64, 2, 4, False, True, True) in configs
+    # independent enumeration of the tile sets
+    tiles = set()
+    for bm, bn, bk, wm, wn, st, epi, direct in itertools.product(
+            (64, 128, 256), (64, 128, 256), (32, 64), (32, 64, 128), (32, 64, 128), (1, 2, 3, 4),
+            (False, True), (False, True)):
+        if bm % wm or bn % wn:
+            continue
+        xcd = ((n // bm) * (n // bn)) % 8 == 0
+        cfg = gm.GemmConfig(bm, bn, bk, wm, wn, st, 1, epi, xcd, direct)
+        try:
+            gm.check_config(cfg, n, n, n)
+        except AssertionError:
+            continue
+        if (n // bm) * (n // bn) < ARCH.sm_nums:
+            continue
+        regs = (gm.est_regs_per_thread(cfg) + 7) // 8 * 8
+        if regs * -(-cfg.num_warps // 4) > 512:
+            continue
+        tiles.add((bm, bn, bk, wm, wn, st, epi, direct))
+    got = {(c.BM, c.BN, c.BK, c.warp_m, c.warp_n, c.stages, c.epi_smem, c.direct) for c in configs}
+    assert got == tiles
+
+
+def test_gemm_rejects_shapes_no_tile_divides():
+    assert Solver.solve_gemm_tc(ARCH, 4096 + 8, 4096, 4096) == []
+
+
+@pytest.mark.parametrize("D,S", [(128, 4096), (64, 4096), (128, 512)])
+def test_flash_attn_configs_are_valid(D, S):
+    B, H = (4, 16) if S == 4096 else (32, 16)
+    configs = Solver.solve_flash_attn(ARCH, B, H, S, S, D)
+    assert configs and len(set(configs)) == len(configs)
+    for cfg in configs:
+        fa.check_config(cfg, S, S, D)
+        assert (S // cfg.Br) * B * H >= ARCH.sm_nums
+    want = set()
+    for br, bc, nw, st in itertools.product((32, 64, 128, 256), (32, 64, 128), (1, 2, 4, 8), (1, 2)):
+        cfg = fa.FAConfig(br, bc, nw, st)
+        try:
+            fa.check_config(cfg, S, S, D)
+        except AssertionError:
+            continue
+        if (S // br) * B * H < ARCH.sm_nums or st > S // bc:
+            continue
+        regs = (fa.est_regs_per_thread(cfg, D) + 7) // 8 * 8
+        if regs * -(-nw // 4) > 512:
+            continue
+        want.add(cfg)
+    assert set(configs) == want
+    # a tighter register budget removes the widest per-wave tiles
+    tight = Solver.solve_flash_attn(ARCH, B, H, S, S, D, max_est_regs=256)
+    assert set(tight) < set(configs) or set(tight) == set(configs)
+    assert all(fa.est_regs_per_thread(c, D) <= 256 for c in tight)
+
+
+def test_z3_backend_agrees_with_enumeration():
+    pytest.importorskip("z3")
+    a = Solver.solve_rowwise(ARCH, "softmax", 16384, 4096, backend="z3")
+    b = Solver.solve_rowwise(ARCH, "softmax", 16384, 4096, backend="enumerate")
+    assert a == b
+    a = Solver.solve_flash_attn(ARCH, 4, 16, 4096, 4096, 128, backend="z3")
+    b = Solver.solve_flash_attn(ARCH, 4, 16, 4096, 4096, 128, backend="enumerate")
+    assert a == b
+
+
+def test_z3_backend_is_reported_missing():
+    if Solver._z3 is not None:
+        pytest.skip("z3 is installed")
+    with pytest.raises(RuntimeError, match="z3"):
+        Solver.solve_rowwise(ARCH, "softmax", 16384, 4096, backend="z3")

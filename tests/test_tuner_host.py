@@ -1,0 +1,159 @@
+"""Host tests of the tuning driver pieces that need no GPU: parallel compile
+with worker failure, record formats, GPU detection, argument parsing."""
+
+import os
+import re
+import sys
+
+import pytest
+
+from deca_amd import Tuner as tuner_mod
+from deca_amd.arch import MI355X
+from deca_amd.kernels.rowwise_hip import RowConfig
+from deca_amd.utils.helper import GPUDetector, byte_size
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+# ---- builders used by the worker pool (must be importable from a spawned process)
+def _ok_builder(tag, path):
+    with open(path, "w") as f:
+        f.write(tag)
+    return path
+
+
+def _dying_builder(tag, path):
+    import multiprocessing
+
+    if tag == "dies" and multiprocessing.current_process().name != "MainProcess":
+        os._exit(3)  # kills the pool worker: the pool breaks
+    return _ok_builder(tag, path)
+
+
+def _failing_builder(tag, path):
+    if tag == "bad":
+        raise RuntimeError("hipcc failed: synthetic error")
+    return _ok_builder(tag, path)
+
+
+def test_build_all_parallel_and_failed_config_is_dropped(capsys):
+    args = {tag: (lambda t: lambda path: (t, path))(tag) for tag in ("a", "bad", "c")}
+    paths = tuner_mod.build_all("test_tuner_host:_failing_builder", args, jobs=2)
+    assert sorted(paths) == ["a", "c"]
+    assert all(open(p).read() == t for t, p in paths.items())
+    assert "bad failed to build" in capsys.readouterr().out
+
+
+def test_build_all_survives_a_dead_worker():
+    """A worker that dies breaks the pool; the affected configs are rebuilt
+    serially in this process (where the builder does not die)."""
+    args = {tag: (lambda t: lambda path: (t, path))(tag) for tag in ("x", "dies", "y")}
+    paths = tuner_mod.build_all("test_tuner_host:_dying_builder", args, jobs=2)
+    assert sorted(paths) == ["dies", "x", "y"]
+    assert open(paths["dies"]).read() == "dies"
+
+
+def test_build_all_serial_when_one_job():
+    args = {"only": lambda path: ("only", path)}
+    assert list(tuner_mod.build_all("test_tuner_host:_ok_builder", args, jobs=1)) == ["only"]
+
+
+class _FakeRowOp:
+    num_bytes = 268435456
+
+    def describe(self):
+        return "Softmax(M=16384, N=4096, float16)"
+
+
+class _FakeGemmOp:
+    num_flops = 2 * 8192**3
+
+    def describe(self):
+        return "GEMMTC(M=8192, N=8192, K=8192, float16)"
+
+
+def test_rowwise_record_format():
+    t = tuner_mod.Tuner("softmax", arch=MI355X(), arch_str="gfx950")
+    msg, best, ref = t._report(_FakeRowOp(), RowConfig(256, 2, 8, hint=True), 3, 24, 42e-6, 84e-6,
+                               1.2e-4, 7.5, 31.0)
+    lines = msg.splitlines()
+    assert re.fullmatch(r"\d{4}-\d\d-\d\d \d\d:\d\d:\d\d \[AMD Instinct MI355X\]", lines[0])
+    assert lines[1] == (" DeCA Softmax(M=16384, N=4096, float16), config: "
+                        "tpr=256,rpb=2,vec=8,mode=reg,hint=1 (cost-model rank 3/24)")
+    assert re.fullmatch(r" throughput: 6391\.3 GB/s \(80% of DRAM peak\), runtime: 0\.0420 ms, "
+                        r"max err: 1\.20e-04", lines[2])
+    assert re.fullmatch(r" torch: 3195\.7 GB/s, runtime: 0\.0840 ms, ratio: 2\.000", lines[3])
+    assert lines[4] == " compile time: 7.5 s, total tuning time: 31.0 s"
+    assert best == pytest.approx(6391.3, abs=0.1) and ref == pytest.approx(3195.7, abs=0.1)
+
+
+def test_gemm_record_format():
+    t = tuner_mod.Tuner("GEMM", arch=MI355X(), arch_str="gfx950")
+    msg, best, _ = t._report(_FakeGemmOp(), "256x256x64,warp=128x64,stages=2,raster=4,epi_smem=0",
+                             1, 24, 0.9e-3, 1.0e-3, 2.4e-4, 20.0, 60.0)
+    assert "throughput: 1221.7 TFLOPS (49% of fp32-acc MFMA peak)" in msg
+    assert "torch: 1099.5 TFLOPS, runtime: 1.0000 ms, ratio: 1.111" in msg
+    assert best == pytest.approx(1221.7, abs=0.1)
+
+
+def test_tuner_rejects_unknown_operator():
+    with pytest.raises(AssertionError):
+        tuner_mod.Tuner("conv2d", arch=MI355X())
+
+
+def test_gpu_lookup_and_detection_failure(capsys):
+    assert GPUDetector.lookup("AMD Radeon Graphics", "gfx950:sramecc+:xnack-") is MI355X
+    assert GPUDetector.lookup("AMD Instinct MI355X", "") is MI355X
+    with pytest.raises(NotImplementedError):
+        GPUDetector.lookup("NVIDIA H20", "sm_90")
+    assert byte_size("float16") == 2 and byte_size("float32") == 4
+    with pytest.raises(ValueError):
+        byte_size("int8")
+
+    class _NoDevice(GPUDetector):
+        @classmethod
+        def _device_info(cls, device_id=0):
+            raise RuntimeError("no HIP device is visible")
+
+    with pytest.raises(SystemExit) as e:
+        _NoDevice.detect_gpu(verbose=True)
+    assert e.value.code == -1
+    assert "GPU detection failed" in capsys.readouterr().out
+
+
+def test_arch_configure_device():
+    class Info:
+        name, gcn_arch = "", "gfx950:sramecc+:xnack-"
+        cu_count, clock_khz, lds_per_block, total_mem = 128, 2000000, 65536, 64 * 2**30
+
+    a = MI355X().configure_device(Info)
+    assert a.name == "AMD Instinct MI355X" and a.gcn_arch == "gfx950"
+    assert a.sm_nums == 128 and a.sm_clock_hz == 2.0e9 and a.max_dyn_smem_per_block == 65536
+    assert a.peak_mma_sync_flops == pytest.approx(128 * 4096 * 2.0)  # GFLOPS
+    base = MI355X()
+    assert base.peak_mma_sync_flops == pytest.approx(2516582, rel=1e-6) and base.dram_bw == 8000
+
+
+def test_driver_argument_parsing():
+    sys.path.insert(0, ROOT)
+    import test_flash_attn
+    import test_gemm_tc
+    import test_rowwise
+
+    a = test_rowwise.parse_args(["--op", "rmsnorm", "--dtype", "bf16", "--shape", "8192", "8192"])
+    assert (a.op, a.dtype, a.shape, a.top_n, a.finalists, a.rounds) == ("rmsnorm", "bf16",
+                                                                      [8192, 8192], 24, 3, 5)
+    g = test_gemm_tc.parse_args(["--sweep"])
+    assert g.sweep and g.shape == [4096, 4096, 4096] and g.top_n == 24
+    f = test_flash_attn.parse_args(["--causal"])
+    assert f.causal and f.top_n == 16 and test_flash_attn.parse_shape(f.shape) == (4, 16, 4096, 4096, 128)
+    assert test_flash_attn.parse_shape([1, 2, 128, 640, 64]) == (1, 2, 128, 640, 64)
+
+
+def test_sweep_csv(tmp_path):
+    import test_gemm_tc
+
+    p = tmp_path / "s.csv"
+    test_gemm_tc.write_sweep_csv([((2048, 2048, 2048), "cfg", 600.0, 500.0)], str(p))
+    assert p.read_text().splitlines() == ["M,N,K,DeCA_TFLOPS,torch_TFLOPS,ratio",
+                                          "2048,2048,2048,600.0000,500.0000,1.2000"]
