@@ -79,18 +79,11 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef __attribute__((address_space(3))) short4v* lds_s4_ptr;
 typedef __attribute__((address_space(3))) void* lptr;
 
-// K tile [BC][D]: 16 consecutive rows at one logical chunk must land on 16
-// different 16-byte bank groups of the 256-byte bank window.
-__device__ __forceinline__ int k_chunk_slot(int row, int c) {
-  constexpr int ROWS_PER_WINDOW = (16 / CPR) > 0 ? (16 / CPR) : 1;
-  constexpr int MASK = (CPR < 16 ? CPR : 16) - 1;
-  return row * CPR + (c ^ ((row / ROWS_PER_WINDOW) & MASK));
-}
-// V tile [BC][D]: the 4 key rows of one transposing read are rotated onto
-// different 64-byte groups.
-__device__ __forceinline__ int v_chunk_slot(int row, int c) {
-  return row * CPR + (c ^ (((row & 3) << 2) & (CPR - 1)));
-}
+// LDS layouts.  K tile [BC][D]: 16-byte chunk c of row r sits at chunk slot
+// c ^ ((r / rows_per_window) & mask), so that 16 consecutive rows at one logical
+// chunk land on 16 different bank groups of the 256-byte bank window.  V tile
+// [BC][D]: chunk c of row r sits at c ^ ((r & 3) << 2), which rotates the 4 key
+// rows of one transposing read onto different 64-byte groups.
 
 #define DECA_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (((n) >> 4) << 14) | 0x0F70)
 
@@ -105,14 +98,22 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
   const int wave_u = __builtin_amdgcn_readfirstlane(wave);
   const int l32 = lane & 31;
   const int half = lane >> 5;
-  const int bh = blockIdx.y;
+  // ---- workgroup -> (batch*head, query tile) ------------------------------------------
+  // 1-D grid.  Workgroups are dealt round-robin to the 8 XCDs; the remap gives
+  // each XCD whole (batch, head) slices, so that the K/V tiles of a slice are
+  // fetched into one L2 only and shared there by all of its query tiles.
+  constexpr int NQ = DECA_SQ / BR;
+  constexpr int TOTAL = NQ * DECA_B * DECA_H;
+  int lin = blockIdx.x;
+  if (TOTAL % 8 == 0) lin = (lin & 7) * (TOTAL / 8) + (lin >> 3);
+  const int bh = lin / NQ;
 #if DECA_CAUSAL
   // Query tiles near the end see the most keys; schedule them first
   // (flash_attn_tir.py:152-156).
-  const int qt = (DECA_SQ / BR - 1) - static_cast<int>(blockIdx.x);
+  const int qt = (NQ - 1) - (lin % NQ);
   const int nkv = ((qt + 1) * BR + BC - 1) / BC;
 #else
-  const int qt = blockIdx.x;
+  const int qt = lin % NQ;
   const int nkv = NKV;
 #endif
   const _Float16* q_base = Q + (static_cast<size_t>(bh) * DECA_SQ + qt * BR + wave * WQ) * D_;
@@ -178,11 +179,25 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
     l_i[mq] = 0.0f;
   }
 
-  // transposing V read: 16-lane block tb, lane ti in the block
+  // ---- LDS read addresses ---------------------------------------------------------------
+  // The swizzles only touch address bits that the loop-varying terms (key block,
+  // d block, k-step) either leave alone or toggle as a whole, so every read is
+  // "per-lane base XOR compile-time constant, plus an immediate offset".
+  // K: row = kt*32 + lane%32, chunk = (ks*2 + half) ^ swz(row); row bits used by
+  // the swizzle do not depend on kt.
+  constexpr int K_RPW = (16 / CPR) > 0 ? (16 / CPR) : 1;
+  constexpr int K_MASK = (CPR < 16 ? CPR : 16) - 1;
+  const unsigned k_lane_base =
+      static_cast<unsigned>(l32 * CPR + (half ^ ((l32 / K_RPW) & K_MASK))) * 16u;
+  static_assert((32 / K_RPW) % (K_MASK + 1) == 0, "K swizzle must not depend on the key block");
+  // V: row = kk*16 + r*8 + (half*4 + ti/4), chunk = (dt*4 + tb%2*2 + ti%4/2) ^ ((row&3) << 2)
   const int tb = lane >> 4, ti = lane & 15;
-  const int v_d_off = 16 * (tb & 1) + 4 * (ti & 3);  // + dt * 32
-  const int v_k_off = (tb >> 1) * 4 + (ti >> 2);     // + kk * 16 + r * 8
-
+  const int v_row0 = (tb >> 1) * 4 + (ti >> 2);
+  const int v_d0 = 16 * (tb & 1) + 4 * (ti & 3);
+  const unsigned v_lane_base = static_cast<unsigned>(
+      v_row0 * CPR * 16 + (((v_d0 >> 3) ^ (((v_row0 & 3) << 2) & (CPR - 1))) * 16) +
+      ((v_d0 >> 2) & 1) * 8);
+  static_assert(CPR >= 8, "D >= 64");
   int slot = 0;
   for (int j = 0; j < nkv; ++j) {
     // Tile j has landed for every lane, and every wave is done with the slot
@@ -209,7 +224,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
 #pragma unroll
       for (int kt = 0; kt < KT; ++kt) {
         const half8 kf = *reinterpret_cast<const half8*>(
-            k_lds + k_chunk_slot(kt * 32 + l32, ks * 2 + half) * 16);
+            k_lds + ((k_lane_base ^ static_cast<unsigned>(ks * 32)) + kt * 32 * CPR * 16));
 #pragma unroll
         for (int mq = 0; mq < MQ; ++mq)
           s_acc[kt][mq] =
@@ -255,7 +270,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
       for (int kt = 0; kt < KT; ++kt) {
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
-          const float p = __builtin_amdgcn_exp2f(s_acc[kt][mq][e] * SL2 - msl);
+          const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s_acc[kt][mq][e], SL2, -msl));
           s_acc[kt][mq][e] = p;
           sum += p;
         }
@@ -294,9 +309,10 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
         half4 h[2];
 #pragma unroll
         for (int r = 0; r < 2; ++r) {
-          const int row = kk * 16 + r * 8 + v_k_off;
-          const int d = dt * 32 + v_d_off;
-          const unsigned char* p = v_lds + v_chunk_slot(row, d >> 3) * 16 + ((d >> 2) & 1) * 8;
+          // d block dt toggles chunk bits 2.. (dt*4); with CPR == 8 only bit 2 is
+          // shared with the swizzle, which the XOR handles as well
+          const unsigned char* p = v_lds + ((v_lane_base ^ static_cast<unsigned>((dt * 4 * 16) & (CPR * 16 - 1))) +
+                                            (kk * 16 + r * 8) * CPR * 16);
           h[r] = __builtin_bit_cast(half4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4_ptr)(p)));
         }
         const half8 vf = __builtin_shufflevector(h[0], h[1], 0, 1, 2, 3, 4, 5, 6, 7);

@@ -91,7 +91,8 @@ def make_flash_attn_fwd(
     softmax_scale: float | None = None, causal: bool = False,
 ) -> KernelSpec:
     """`causal` applies the top-left aligned mask (key j visible to query i iff j <= i).
-    Grid (S_q / Br, B * H), block `threads` (reference: flash_attn_tir.py:147)."""
+    1-D grid of (S_q / Br) * B * H workgroups (reference: 2-D, flash_attn_tir.py:147; the
+    kernel remaps ids so that each XCD owns whole (batch, head) slices), block `threads`."""
     check_config(cfg, S_q, S_kv, D)
     assert not causal or S_q == S_kv, "causal attention requires S_q == S_kv"
     scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(D)
@@ -102,7 +103,7 @@ def make_flash_attn_fwd(
         "DECA_SCALE": repr(float(scale)),
     }
     return make_spec(
-        TEMPLATE, defines, grid=(S_q // cfg.Br, B * H, 1), block=(cfg.threads, 1, 1), nargs=4,
+        TEMPLATE, defines, grid=((S_q // cfg.Br) * B * H, 1, 1), block=(cfg.threads, 1, 1), nargs=4,
         options=FAST_MATH_OPTIONS, meta={"cfg": str(cfg), "causal": causal},
     )
 
