@@ -11,6 +11,8 @@
 //   DECA_STAGES         K/V LDS ring depth (1 or 2)
 //   DECA_CAUSAL         1: key j visible to query i iff j <= i (SQ == SKV)
 //   DECA_SCALE          softmax scale
+//   DECA_PIPE           1: S^T of the next tile is computed before the softmax of
+//                       the current one (two S^T accumulators per wave)
 //
 // The problem is computed transposed, which is what makes the two MFMA
 // products chain without a layout change on CDNA:
@@ -143,18 +145,18 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
                  : "v"(voff), "s"(origin), "s"(lds_addr)
                  : "memory");
   };
-  auto issue_tile = [&](int j, int slot) {
-    const _Float16* k_origin = k_base + static_cast<size_t>(j) * BC * D_;
-    const _Float16* v_origin = v_base + static_cast<size_t>(j) * BC * D_;
-    const unsigned k_dst = lds_u + slot * TILE_BYTES + wave_u * 1024;
-    const unsigned v_dst = lds_u + (STAGES + slot) * TILE_BYTES + wave_u * 1024;
+  auto issue_k = [&](int j, int slot) {
+    const _Float16* origin = k_base + static_cast<size_t>(j) * BC * D_;
+    const unsigned dst = lds_u + slot * TILE_BYTES + wave_u * 1024;
 #pragma unroll
-    for (int it = 0; it < KV_IT; ++it) dma16(k_origin, k_voff[it], k_dst + it * NT * 16);
-#pragma unroll
-    for (int it = 0; it < KV_IT; ++it) dma16(v_origin, v_voff[it], v_dst + it * NT * 16);
+    for (int it = 0; it < KV_IT; ++it) dma16(origin, k_voff[it], dst + it * NT * 16);
   };
-
-  issue_tile(0, 0);
+  auto issue_v = [&](int j, int slot) {
+    const _Float16* origin = v_base + static_cast<size_t>(j) * BC * D_;
+    const unsigned dst = lds_u + (STAGES + slot) * TILE_BYTES + wave_u * 1024;
+#pragma unroll
+    for (int it = 0; it < KV_IT; ++it) dma16(origin, v_voff[it], dst + it * NT * 16);
+  };
 
   // ---- Q fragments: VGPR resident for the whole kernel ----------------------------
   // lane (q = lane % 32, half): 8 consecutive d at ks * 16 + half * 8
@@ -198,21 +200,10 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
       v_row0 * CPR * 16 + (((v_d0 >> 3) ^ (((v_row0 & 3) << 2) & (CPR - 1))) * 16) +
       ((v_d0 >> 2) & 1) * 8);
   static_assert(CPR >= 8, "D >= 64");
-  int slot = 0;
-  for (int j = 0; j < nkv; ++j) {
-    // Tile j has landed for every lane, and every wave is done with the slot
-    // that tile j+1 is about to overwrite.
-    DECA_WAIT_VMCNT(0);
-    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wave's LDS reads have returned
-    __builtin_amdgcn_s_barrier();
-#if STAGES == 2
-    if (j + 1 < nkv) issue_tile(j + 1, slot ^ 1);
-#endif
-    const unsigned char* k_lds = lds + slot * TILE_BYTES;
-    const unsigned char* v_lds = lds + (STAGES + slot) * TILE_BYTES;
-
-    // ---- S^T = K Q^T ----------------------------------------------------------------
-    floatx16 s_acc[KT][MQ];
+  // ---- the three phases of one KV step ----------------------------------------------------
+  // S^T = K Q^T for the tile in K slot `kslot`
+  auto compute_s = [&](floatx16 (&s_acc)[KT][MQ], int kslot) {
+    const unsigned char* k_lds = lds + kslot * TILE_BYTES;
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
@@ -231,10 +222,12 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
               __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[mq][ks], s_acc[kt][mq], 0, 0, 0);
       }
     }
-
+  };
+  // Causal mask of tile j.  Only tiles crossing the diagonal need it; every
+  // query sees key 0 in tile 0, so its running max is finite before a fully
+  // masked block shows up.
+  auto mask_s = [&](floatx16 (&s_acc)[KT][MQ], int j) {
 #if DECA_CAUSAL
-    // Only tiles crossing the diagonal need masking.  Every query sees key 0 in
-    // tile 0, so its running max is finite before a fully masked block shows up.
     if ((j + 1) * BC - 1 > qt * BR + wave * WQ) {
 #pragma unroll
       for (int mq = 0; mq < MQ; ++mq) {
@@ -248,10 +241,15 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
           }
       }
     }
+#else
+    (void)s_acc;
+    (void)j;
 #endif
-
-    // ---- online softmax: one query column per lane ------------------------------------
-    half8 pf[KK][MQ];
+  };
+  // Online softmax of one tile: one query column per lane.  Leaves P^T (fp16,
+  // already in operand order) in `pf` and rescales O^T when a running max moved
+  // (skipped otherwise: multiplying by 1 is exact).
+  auto softmax = [&](floatx16 (&s_acc)[KT][MQ], half8 (&pf)[KK][MQ]) {
     float alpha[MQ];
 #pragma unroll
     for (int mq = 0; mq < MQ; ++mq) {
@@ -284,24 +282,23 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
       }
       l_i[mq] = l_i[mq] * alpha[mq] + sum;
     }
-    // O^T *= alpha (skipped when no running max moved: multiplying by 1 is exact)
-    {
-      bool moved = false;
+    bool moved = false;
 #pragma unroll
-      for (int mq = 0; mq < MQ; ++mq) moved |= (alpha[mq] != 1.0f);
-      if (__builtin_amdgcn_ballot_w64(moved) != 0) {
+    for (int mq = 0; mq < MQ; ++mq) moved |= (alpha[mq] != 1.0f);
+    if (__builtin_amdgcn_ballot_w64(moved) != 0) {
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
+      for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-          for (int mq = 0; mq < MQ; ++mq)
+        for (int mq = 0; mq < MQ; ++mq)
 #pragma unroll
-            for (int e = 0; e < 16; ++e) o_acc[dt][mq][e] *= alpha[mq];
-      }
+          for (int e = 0; e < 16; ++e) o_acc[dt][mq][e] *= alpha[mq];
     }
-
-    // ---- O^T += V^T P^T ----------------------------------------------------------------
-    // k-slot (half, e) of step kk is key row kk*16 + (e/4)*8 + half*4 + e%4: the
-    // order in which the S^T accumulator registers hold the keys.
+  };
+  // O^T += V^T P^T for the tile in V slot `vslot`.  k-slot (half, e) of step kk
+  // is key row kk*16 + (e/4)*8 + half*4 + e%4: the order in which the S^T
+  // accumulator registers hold the keys.
+  auto compute_pv = [&](const half8 (&pf)[KK][MQ], int vslot) {
+    const unsigned char* v_lds = lds + (STAGES + vslot) * TILE_BYTES;
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) {
 #pragma unroll
@@ -309,10 +306,9 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
         half4 h[2];
 #pragma unroll
         for (int r = 0; r < 2; ++r) {
-          // d block dt toggles chunk bits 2.. (dt*4); with CPR == 8 only bit 2 is
-          // shared with the swizzle, which the XOR handles as well
-          const unsigned char* p = v_lds + ((v_lane_base ^ static_cast<unsigned>((dt * 4 * 16) & (CPR * 16 - 1))) +
-                                            (kk * 16 + r * 8) * CPR * 16);
+          const unsigned char* p =
+              v_lds + ((v_lane_base ^ static_cast<unsigned>((dt * 4 * 16) & (CPR * 16 - 1))) +
+                       (kk * 16 + r * 8) * CPR * 16);
           h[r] = __builtin_bit_cast(half4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4_ptr)(p)));
         }
         const half8 vf = __builtin_shufflevector(h[0], h[1], 0, 1, 2, 3, 4, 5, 6, 7);
@@ -322,16 +318,193 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
               __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf[kk][mq], o_acc[dt][mq], 0, 0, 0);
       }
     }
+  };
+  auto wait_and_barrier = [&]() {
+    DECA_WAIT_VMCNT(0);                  // this lane's outstanding tile loads have landed
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wave's LDS reads have returned
+    __builtin_amdgcn_s_barrier();
+  };
 
+#if DECA_PIPE
+  // ---- software-pipelined loop ------------------------------------------------------------
+  // S^T of tile j+1 is computed in the same straight-line block as the
+  // exponentials and the second product of tile j, so that one wave's matrix
+  // work overlaps its own vector work.  The row statistics (max, rescale factor)
+  // of a tile are taken as soon as its S^T is complete, one iteration before its
+  // exponentials, which moves the data-dependent O^T rescale (a branch) to the
+  // top of the iteration and leaves the rest branch-free.
+  // Iteration j needs K_{j+1} and V_j in LDS; both were requested during
+  // iteration j-1.  K tile t and V tile t live in slot t % 2 of their rings.
+  static_assert(STAGES == 2, "the pipelined loop uses two K and two V slots");
+  float alpha[MQ], msl[MQ];
+  // m' = max(m, rowmax S); alpha = exp2((m - m') * sl2); msl = m' * sl2
+  auto row_stats = [&](const floatx16 (&s_acc)[KT][MQ]) {
+#pragma unroll
+    for (int mq = 0; mq < MQ; ++mq) {
+      float mx = s_acc[0][mq][0];
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) mx = fmaxf(mx, s_acc[kt][mq][e]);
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float m_new = fmaxf(m_i[mq], mx);
+      alpha[mq] = __builtin_amdgcn_exp2f((m_i[mq] - m_new) * SL2);
+      m_i[mq] = m_new;
+      msl[mq] = m_new * SL2;
+    }
+  };
+  auto rescale_o = [&]() {
+    bool moved = false;
+#pragma unroll
+    for (int mq = 0; mq < MQ; ++mq) moved |= (alpha[mq] != 1.0f);
+    if (__builtin_amdgcn_ballot_w64(moved) != 0) {
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int mq = 0; mq < MQ; ++mq)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) o_acc[dt][mq][e] *= alpha[mq];
+    }
+  };
+  // p = exp2(S * sl2 - msl); l = l * alpha + sum p; P = fp16(p) in operand order
+  auto exp_and_pack = [&](floatx16 (&s_acc)[KT][MQ], half8 (&pf)[KK][MQ]) {
+#pragma unroll
+    for (int mq = 0; mq < MQ; ++mq) {
+      float sum = 0.0f;
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s_acc[kt][mq][e], SL2, -msl[mq]));
+          s_acc[kt][mq][e] = p;
+          sum += p;
+        }
+#pragma unroll
+        for (int hh = 0; hh < 2; ++hh) {
+          half8 h;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) h[e] = static_cast<_Float16>(s_acc[kt][mq][hh * 8 + e]);
+          pf[kt * 2 + hh][mq] = h;
+        }
+      }
+      l_i[mq] = l_i[mq] * alpha[mq] + sum;
+    }
+  };
+  // S^T of the next tile (K slot `kslot`) fused with the exponentials of the
+  // current one: after the MFMAs of step (ks, kt) a fixed share of the current
+  // tile's scores is exponentiated, and nothing is allowed to move across the
+  // step boundary, so the matrix pipe and the vector ALU stay busy together.
+  auto s_next_and_exp = [&](floatx16 (&s_nxt)[KT][MQ], floatx16 (&s_cur)[KT][MQ],
+                            half8 (&pf)[KK][MQ], int kslot) {
+    const unsigned char* k_lds = lds + kslot * TILE_BYTES;
+    constexpr int STEPS = DK * KT;
+    constexpr int EPS_ = (KT * 16) / STEPS;  // scores of the current tile per step and q tile
+    static_assert((KT * 16) % STEPS == 0 && EPS_ >= 1, "scores must divide over the steps");
+    const floatx16 zero = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f,
+                           0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    float sum[MQ];
+#pragma unroll
+    for (int mq = 0; mq < MQ; ++mq) sum[mq] = 0.0f;
+    half8 kf_next = *reinterpret_cast<const half8*>(k_lds + k_lane_base);
+#pragma unroll
+    for (int step = 0; step < STEPS; ++step) {
+      const int ks = step / KT, kt = step % KT;
+      const half8 kf = kf_next;
+      if (step + 1 < STEPS) {
+        const int ks1 = (step + 1) / KT, kt1 = (step + 1) % KT;
+        kf_next = *reinterpret_cast<const half8*>(
+            k_lds + ((k_lane_base ^ static_cast<unsigned>(ks1 * 32)) + kt1 * 32 * CPR * 16));
+      }
+#pragma unroll
+      for (int mq = 0; mq < MQ; ++mq)
+        s_nxt[kt][mq] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+            kf, qf[mq][ks], ks == 0 ? zero : s_nxt[kt][mq], 0, 0, 0);
+#pragma unroll
+      for (int mq = 0; mq < MQ; ++mq)
+#pragma unroll
+        for (int i = 0; i < EPS_; ++i) {
+          const int lin = step * EPS_ + i, ct = lin / 16, ce = lin % 16;
+          const float p =
+              __builtin_amdgcn_exp2f(__builtin_fmaf(s_cur[ct][mq][ce], SL2, -msl[mq]));
+          s_cur[ct][mq][ce] = p;
+          sum[mq] += p;
+          if (lin % 8 == 7) {  // an 8-key block is complete: pack it in operand order
+            half8 h;
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+              h[e] = static_cast<_Float16>(s_cur[ct][mq][(ce / 8) * 8 + e]);
+            pf[ct * 2 + ce / 8][mq] = h;
+          }
+        }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int mq = 0; mq < MQ; ++mq) l_i[mq] = l_i[mq] * alpha[mq] + sum[mq];
+  };
+
+  issue_k(0, 0);
+  issue_v(0, 0);
+  if (nkv > 1) issue_k(1, 1);
+  floatx16 s_cur[KT][MQ], s_nxt[KT][MQ];
+  half8 pf[KK][MQ];
+  wait_and_barrier();
+  compute_s(s_cur, 0);
+  mask_s(s_cur, 0);
+  row_stats(s_cur);
+  for (int j = 0; j < nkv - 1; ++j) {
+    const int cur = j & 1;
+    wait_and_barrier();  // K_{j+1}, V_j landed; everyone is done with K_j and V_{j-1}
+    if (j + 2 < nkv) issue_k(j + 2, cur);
+    issue_v(j + 1, cur ^ 1);
+    rescale_o();
+    // -- matrix and vector work of two different tiles, interleaved step by step --
+    s_next_and_exp(s_nxt, s_cur, pf, cur ^ 1);
+    compute_pv(pf, cur);
+    mask_s(s_nxt, j + 1);
+    row_stats(s_nxt);
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+      for (int mq = 0; mq < MQ; ++mq) s_cur[kt][mq] = s_nxt[kt][mq];
+  }
+  // last tile: nothing left to prefetch
+  wait_and_barrier();
+  rescale_o();
+  exp_and_pack(s_cur, pf);
+  compute_pv(pf, (nkv - 1) & 1);
+#else
+  issue_k(0, 0);
+  issue_v(0, 0);
+  int slot = 0;
+  for (int j = 0; j < nkv; ++j) {
+    // Tile j has landed for every lane, and every wave is done with the slot
+    // that tile j+1 is about to overwrite.
+    wait_and_barrier();
+#if STAGES == 2
+    if (j + 1 < nkv) {
+      issue_k(j + 1, slot ^ 1);
+      issue_v(j + 1, slot ^ 1);
+    }
+#endif
+    floatx16 s_acc[KT][MQ];
+    half8 pf[KK][MQ];
+    compute_s(s_acc, slot);
+    mask_s(s_acc, j);
+    softmax(s_acc, pf);
+    compute_pv(pf, slot);
 #if STAGES == 2
     slot ^= 1;
 #else
     // single slot: everyone must be done reading before the refill
     __builtin_amdgcn_s_waitcnt(0xC07F);
     __builtin_amdgcn_s_barrier();
-    if (j + 1 < nkv) issue_tile(j + 1, 0);
+    if (j + 1 < nkv) {
+      issue_k(j + 1, 0);
+      issue_v(j + 1, 0);
+    }
 #endif
   }
+#endif
 
   // ---- epilogue: O[q][d] = O^T[d][q] / l ----------------------------------------------
   // o_acc[dt][mq][e]: q = mq*32 + lane%32, d = dt*32 + (e/4)*8 + half*4 + e%4

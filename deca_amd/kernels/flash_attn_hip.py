@@ -40,6 +40,7 @@ class FAConfig:
     stages: int = 2  # K/V LDS ring depth
     q_in_smem: bool = False  # kept for the record format; Q always lives in VGPRs here
     swizzle: bool = True  # kept for the record format; the LDS layout is always swizzled
+    pipe: bool = False  # compute S^T of tile j+1 before the softmax of tile j
 
     @property
     def threads(self) -> int:
@@ -52,6 +53,7 @@ class FAConfig:
         return (
             f"Br={self.Br},Bc={self.Bc},warps={self.num_warps},stages={self.stages},"
             f"q_smem={int(self.q_in_smem)},swz={int(self.swizzle)}"
+            + (",pipe=1" if self.pipe else "")
         )
 
 
@@ -66,6 +68,8 @@ def est_regs_per_thread(cfg: FAConfig, D: int) -> int:
     o_acc = (D // 32) * mq * 16
     s_acc = (cfg.Bc // 32) * mq * 16
     p_h = s_acc // 2
+    if cfg.pipe:
+        s_acc *= 2
     q_frag = mq * (D // 16) * 4
     kv_frag = 2 * 4 * 2  # a few K / V fragments in flight
     return o_acc + s_acc + p_h + q_frag + kv_frag + 4 * mq + 40
@@ -81,6 +85,7 @@ def check_config(cfg: FAConfig, S_q: int, S_kv: int, D: int) -> None:
     assert 2 * (cfg.Bc * cpr) // cfg.threads <= 63
     assert cfg.threads <= 1024
     assert cfg.stages in (1, 2)
+    assert not cfg.pipe or cfg.stages == 2
     assert not cfg.q_in_smem and cfg.swizzle
     assert smem_bytes(cfg, D) <= MAX_LDS
     assert est_regs_per_thread(cfg, D) <= 512
@@ -100,7 +105,7 @@ def make_flash_attn_fwd(
         "DECA_B": B, "DECA_H": H, "DECA_SQ": S_q, "DECA_SKV": S_kv, "DECA_D": D,
         "DECA_BR": cfg.Br, "DECA_BC": cfg.Bc, "DECA_NW": cfg.num_warps,
         "DECA_STAGES": cfg.stages, "DECA_CAUSAL": int(causal),
-        "DECA_SCALE": repr(float(scale)),
+        "DECA_SCALE": repr(float(scale)), "DECA_PIPE": int(cfg.pipe),
     }
     return make_spec(
         TEMPLATE, defines, grid=((S_q // cfg.Br) * B * H, 1, 1), block=(cfg.threads, 1, 1), nargs=4,

@@ -101,6 +101,12 @@ FA_CASES = [
     (1, 3, 128, 640, 128, False, FAConfig(64, 64, 2, 2)),   # S_q != S_kv
     (1, 1, 384, 128, 64, False, FAConfig(128, 128, 4, 1)),
     (1, 1, 128, 128, 128, True, FAConfig(32, 32, 1, 2)),
+    # S^T computed one tile ahead of the softmax
+    (1, 2, 512, 512, 128, False, FAConfig(256, 64, 8, 2, pipe=True)),
+    (1, 2, 512, 512, 128, True, FAConfig(256, 64, 8, 2, pipe=True)),
+    (2, 2, 512, 512, 64, True, FAConfig(128, 128, 4, 2, pipe=True)),
+    (1, 2, 256, 384, 128, False, FAConfig(128, 128, 4, 2, pipe=True)),
+    (1, 1, 128, 64, 64, False, FAConfig(64, 64, 2, 2, pipe=True)),   # a single KV tile
 ]
 
 FA_FULL = [
