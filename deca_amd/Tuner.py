@@ -218,7 +218,8 @@ class Tuner:
                 print(rt.record, flush=True)
                 res.append((rt.throughput, cfg, rt.execution_time, rt.max_error))
             except Exception as e:  # noqa: BLE001
-                print(f"{cfg} is not a valid config: {str(e)[-200:]}", flush=True)
+                text = str(e) if os.environ.get("DECA_VERBOSE") else str(e)[-200:]
+                print(f"{cfg} is not a valid config: {text}", flush=True)
             finally:
                 if rt.runtime_mod is not None:
                     rt.runtime_mod.close()

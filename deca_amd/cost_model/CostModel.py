@@ -48,29 +48,35 @@ def rowwise_score(cfg, arch, op: str, M: int, N: int, type_size: int = 2) -> flo
       row is requested up front in `reg` mode, `unroll` chunks in `twopass`)
       against Little's law, HBM bandwidth per CU x latency under load
       (`arch.dram_latency_s`)
-    - phases: a workgroup loads, reduces, then stores; with few resident
-      workgroups per CU the reduce/store phase is not hidden by other loads
-    - wave efficiency of the grid of M / rows_per_block workgroups
+    - granularity: a wave can only start reducing once all of its chunks have
+      arrived and stores nothing until the row is reduced, so long per-lane chunk
+      lists (few lanes per row) serialise load, math and store inside each wave;
+      measured on MI355X the sweet spot is two 16-byte chunks per lane
+    - wave efficiency of the grid of M / rows_per_block workgroups, and the
+      drain bubble of large workgroups (all waves of a workgroup retire
+      together, so 1024-lane workgroups leave wave slots idle at their tails)
     - twopass re-reads the row; the re-read hits L2 / Infinity Cache when the
       rows in flight fit
-    - rows spanning several waves pay an LDS exchange and a barrier per
-      reduction; rows narrower than a wave idle no lanes but shorten bursts
+    - rows spanning several waves pay an LDS exchange and a barrier per reduction
     - idle vector lanes of the last chunk (tail) and 8-byte accesses
-    - non-temporal accesses keep the streamed data from displacing reusable lines
+    - non-temporal accesses: streamed data does not displace lines in L2 /
+      Infinity Cache and the writes drain earlier (measured: ~8% on MI355X)
     """
     from deca_amd.kernels.rowwise_hip import num_chunks
 
     wgs = rowwise_occupancy(cfg, arch, op, N)
     chunks = num_chunks(cfg, N)
-    per_lane = (chunks if cfg.mode == "reg" else cfg.unroll) * cfg.vec * type_size
-    in_flight = wgs * cfg.threads * per_lane
+    depth = chunks if cfg.mode == "reg" else cfg.unroll
+    in_flight = wgs * cfg.threads * depth * cfg.vec * type_size
     need = arch.dram_bw * 1e9 / arch.sm_nums * getattr(arch, "dram_latency_s", 2e-6)
     mem = min(1.0, in_flight / need)
 
-    phase = 1.0 - (0.35 if cfg.mode == "reg" else 0.1) / wgs
+    granularity = 1.0 / (1.0 + 0.012 * max(0, depth - 2)) * (0.985 if depth == 1 else 1.0)
 
     grid = M // cfg.rows_per_block
     wave_eff = _wave_efficiency(grid, arch.sm_nums * wgs)
+    drain = 1.0 / (1.0 + 0.10 * max(0.0, cfg.threads / 256 - 2.0))
+    rows = 1.0 / (1.0 + 0.015 * abs(math.log2(cfg.rows_per_block) - 1.0))
 
     passes = 1.0
     if cfg.mode == "twopass":
@@ -81,15 +87,16 @@ def rowwise_score(cfg, arch, op: str, M: int, N: int, type_size: int = 2) -> flo
         passes = 1.0 + 0.5 * (hit * arch.dram_bw / reread_bw + (1.0 - hit))
 
     waves_per_row = max(1, cfg.threads_per_row // arch.warp_size)
-    reduce = 1.0 / (1.0 + 0.02 * math.log2(waves_per_row) + (0.03 if waves_per_row > 1 else 0.0))
+    reduce = 1.0 / (1.0 + 0.005 * math.log2(waves_per_row))
     if cfg.threads_per_row < arch.warp_size:
         reduce *= 0.97
 
     tail = N / (chunks * cfg.threads_per_row * cfg.vec) if cfg.mode == "reg" else 1.0
-    lanes = 1.0 if cfg.vec * type_size >= 16 else 0.97
-    stream = 1.0 if cfg.hint else getattr(arch, "rowwise_no_hint_factor", 0.96)
+    lanes = 1.0 if cfg.vec * type_size >= 16 else 0.985
+    stream = 1.0 if cfg.hint else getattr(arch, "rowwise_no_hint_factor", 0.92)
 
-    return mem * phase * wave_eff * reduce * (0.7 + 0.3 * tail) * lanes * stream / passes
+    return (mem * granularity * wave_eff * drain * rows * reduce * (0.7 + 0.3 * tail) * lanes *
+            stream / passes)
 
 
 def rank_rowwise_configs(configs, arch, op: str, M: int, N: int, top_n: int | None = None):

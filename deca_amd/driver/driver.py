@@ -92,6 +92,15 @@ class HipDriver:
                 f"{lib_path} is missing: build it with `python -m deca_amd.driver.build_lib` "
                 "(there is no fallback path without the HIP launcher library)"
             )
+        # torch ships its own copy of the HIP runtime under the same soname
+        # (libamdhip64.so.7).  Tensors come from torch, so its runtime must be the
+        # one in the process: import it before this library is mapped, otherwise
+        # the system copy is loaded first and torch later finds "no ROCm-capable
+        # device".
+        try:
+            import torch  # noqa: F401
+        except ImportError:  # the library also works standalone (raw device pointers)
+            pass
         self.lib = ctypes.CDLL(lib_path)
         for name, (restype, argtypes) in C_API.items():
             fn = getattr(self.lib, name)

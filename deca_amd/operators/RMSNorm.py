@@ -1,22 +1,6 @@
-"""
-RMSNorm over the last dimension of an [M, N] tensor with a weight (forward):
-y = x * rsqrt(mean(x^2) + eps) * w
-"""
+"""RMSNorm over the last dimension of an [M, N] tensor (defined with the other
+row-wise operators; kept as a module for `from operators.RMSNorm import RMSNorm`)."""
 
-from deca_amd.operators.Rowwise import RowwiseOperator
+from deca_amd.operators.Rowwise import RMSNorm  # noqa: F401
 
-
-class RMSNorm(RowwiseOperator):
-    op_kind = "rmsnorm"
-
-    def __init__(
-        self, M: int, N: int, dtype: str = "float16", eps: float = 1e-6, name: str = "RMSNorm"
-    ):
-        """
-        Args:
-            M: number of rows (tokens)
-            N: hidden size
-            dtype: "float16" or "bfloat16" (fp32 math)
-            eps: added to the mean square
-        """
-        super().__init__(M, N, dtype, eps, name=name)
+__all__ = ["RMSNorm"]

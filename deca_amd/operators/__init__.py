@@ -1,6 +1,9 @@
-from .Op import *  # noqa: F401,F403
-from .GEMMTC import *  # noqa: F401,F403
-from .FlashAttention import *  # noqa: F401,F403
-from .Rowwise import *  # noqa: F401,F403
-from .Softmax import *  # noqa: F401,F403
-from .RMSNorm import *  # noqa: F401,F403
+"""Operator descriptors: shape, work count, inputs, reference, tolerance and the
+kernel specialisation of a config."""
+
+from .FlashAttention import FlashAttention
+from .GEMMTC import GEMMTC
+from .Op import Operator
+from .Rowwise import RMSNorm, RowwiseOperator, Softmax
+
+__all__ = ["Operator", "RowwiseOperator", "Softmax", "RMSNorm", "GEMMTC", "FlashAttention"]
