@@ -77,6 +77,7 @@ class MI355X(Arch):
 
         # ---- fitted penalties read via getattr by the cost model ---------------------
         self.gemm_excess_stage_penalty = 0.02
+        self.gemm_fill_latency_s = 0.75e-6
         self.fa_cta_sync_penalty = 0.05
 
         self.bandwidth = [self.dram_bw, self.smem_bw_per_sm * self.sm_nums / 1e9]

@@ -158,7 +158,8 @@ def gemm_tc_score(cfg, arch, M: int, N: int, K: int) -> float:
       latency before the first MFMA of a k-step, the barrier); a second wave does
     - pipelining: bytes in flight ((stages - 1) tiles per workgroup, or one tile
       for the VGPR-staged ring) vs. Little's law on the L2 stream; excess
-      stages are penalised by `arch.gemm_excess_stage_penalty`
+      stages are penalised by `arch.gemm_excess_stage_penalty` (fitted on MI355X:
+      a window of one 64-deep tile already saturates; deeper rings cost ~2% each)
     - one barrier per BK stage
     - epilogue: C is written once; direct stores are 8-byte row segments, the
       staged epilogue writes 16-byte coalesced chunks
@@ -185,8 +186,9 @@ def gemm_tc_score(cfg, arch, M: int, N: int, K: int) -> float:
     terms = sorted([t_mma, t_lds, t_l2, t_dram])
     t_flop = terms[-1] + 0.25 * sum(terms[:-1])
 
-    # Bytes per CU that must be in flight to cover ~1.5 us of L2 / fabric latency.
-    need = fill_bpf / t_mma * 1.5e-6
+    # Bytes per CU that must be in flight to cover the L2 / fabric latency at the
+    # sustained (power-limited, about half of peak) MFMA rate: ~0.75 us at peak rate.
+    need = fill_bpf / t_mma * getattr(arch, "gemm_fill_latency_s", 0.75e-6)
     stage_bytes = wgs * (cfg.BM + cfg.BN) * cfg.BK * 2
     depth = (cfg.stages - 1) if cfg.direct else 1
     in_flight = max(depth, 0.5) * stage_bytes
@@ -194,16 +196,20 @@ def gemm_tc_score(cfg, arch, M: int, N: int, K: int) -> float:
     excess = max(0, depth - math.ceil(need / stage_bytes))
     pipe *= 1.0 - getattr(arch, "gemm_excess_stage_penalty", 0.0) * excess
 
-    # CU cycles per stage at the MFMA rate vs. ~200 cycles of barrier + refill issue
+    # CU cycles per stage at the MFMA rate vs. ~100 cycles of barrier + refill issue
     flops_per_cycle = peak * 1e9 / cus / arch.sm_clock_hz
     stage_cycles = 2 * cfg.BM * cfg.BN * cfg.BK / flops_per_cycle
-    sync_eff = 1.0 / (1.0 + 200.0 / wgs / stage_cycles)
+    sync_eff = 1.0 / (1.0 + 100.0 / wgs / stage_cycles)
 
     epi_eff = 1.0 if cfg.epi_smem else 0.5
     t_epi = (1.0 / K) / epi_eff * cus / (arch.dram_bw * 1e9)
     t_epi *= 1.0 if wgs == 1 else 0.4
 
-    return wave_eff * hiding * pipe * sync_eff / ((t_flop + t_epi) / t_mma)
+    # VGPR-staged fills add global-load, LDS-write and wait instructions to the
+    # MFMA issue stream (measured ~15% on MI355X)
+    staged = 1.0 if cfg.direct else getattr(arch, "gemm_staged_fill_factor", 0.85)
+
+    return wave_eff * hiding * pipe * sync_eff * staged / ((t_flop + t_epi) / t_mma)
 
 
 def rank_gemm_configs(configs, arch, M: int, N: int, K: int, top_n: int | None = None):
