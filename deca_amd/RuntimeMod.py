@@ -84,15 +84,20 @@ class RuntimeMod:
 
     # ---- verification --------------------------------------------------------------------
     def _errors(self, out, ref, atol: float, rtol: float):
-        """(max |out - ref|, max |out - ref| / (atol + rtol |ref|)) in row blocks."""
+        """(max |out - ref|, max |out - ref| / (atol + rtol |ref|)) in row blocks.
+        A NaN anywhere in the output makes both infinite (Python's max() would
+        otherwise drop it and let a broken kernel pass)."""
         out2, ref2 = out.reshape(-1, out.shape[-1]), ref.reshape(-1, ref.shape[-1])
         step = max(1, _VERIFY_ELEMS // ref2.shape[-1])
         worst, excess = 0.0, 0.0
         for r0 in range(0, ref2.shape[0], step):
             r = ref2[r0 : r0 + step].float()
             d = (out2[r0 : r0 + step].float() - r).abs()
-            worst = max(worst, d.max().item())
-            excess = max(excess, (d / (atol + rtol * r.abs())).max().item())
+            block_worst = d.max().item()
+            block_excess = (d / (atol + rtol * r.abs())).max().item()
+            if block_worst != block_worst or block_excess != block_excess:  # NaN
+                return float("inf"), float("inf")
+            worst, excess = max(worst, block_worst), max(excess, block_excess)
         return worst, excess
 
     def _measure(self, verify: bool, abs_tol: float | None):

@@ -157,3 +157,27 @@ def test_sweep_csv(tmp_path):
     test_gemm_tc.write_sweep_csv([((2048, 2048, 2048), "cfg", 600.0, 500.0)], str(p))
     assert p.read_text().splitlines() == ["M,N,K,DeCA_TFLOPS,torch_TFLOPS,ratio",
                                           "2048,2048,2048,600.0000,500.0000,1.2000"]
+
+
+def test_runtime_mod_error_metric_and_nan():
+    """The verification metric on host tensors: max |d|, the reference's
+    excess ratio, and NaN outputs counted as failures."""
+    import torch
+
+    from deca_amd.RuntimeMod import RuntimeMod
+
+    rt = RuntimeMod(_FakeRowOp(), MI355X(), False, RowConfig())
+    ref = torch.tensor([[1.0, -2.0, 0.0, 4.0]])
+    out = ref + torch.tensor([[0.001, 0.0, 0.0, -0.004]])
+    worst, excess = rt._errors(out, ref, 1e-2, 2e-3)
+    assert worst == pytest.approx(0.004, rel=1e-3)
+    assert excess == pytest.approx(0.004 / (1e-2 + 2e-3 * 4), rel=1e-3)
+    bad = out.clone()
+    bad[0, 1] = float("nan")
+    assert rt._errors(bad, ref, 1e-2, 2e-3) == (float("inf"), float("inf"))
+    # 4-D attention outputs are compared through the same row-block loop
+    o4 = torch.zeros(2, 3, 5, 8)
+    assert rt._errors(o4 + 0.5, o4, 1.0, 0.0) == (0.5, 0.5)
+    with pytest.raises(RuntimeError, match="no kernel loaded"):
+        rt.time_kernel_op()
+    assert rt.is_flash_attn is False
