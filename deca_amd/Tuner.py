@@ -109,7 +109,7 @@ class Tuner:
         from deca_amd import operators as ops
 
         if self.operator == "GEMM":
-            return ops.GEMMTC(*shape)
+            return ops.GEMMTC(*shape, dtype=dtype)
         if self.operator == "softmax":
             return ops.Softmax(*shape, dtype)
         if self.operator == "rmsnorm":
@@ -139,7 +139,7 @@ class Tuner:
         """(function path, cfg -> (path -> args))."""
         if self.operator == "GEMM":
             return ("deca_amd.kernels.gemm_hip:build_gemm_tc_to_file",
-                    lambda cfg: lambda path: (tuple(shape), cfg, self.arch_str, path))
+                    lambda cfg: lambda path: (tuple(shape), cfg, self.arch_str, path, op.dtype))
         if self.operator in ("softmax", "rmsnorm"):
             return ("deca_amd.kernels.rowwise_hip:build_rowwise_to_file",
                     lambda cfg: lambda path: (self.operator, tuple(shape), op.dtype, cfg, op.eps,

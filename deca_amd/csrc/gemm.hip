@@ -1,5 +1,6 @@
-// fp16 x fp16 -> fp32-accumulate GEMM, C[M,N] = A[M,K] * B[K,N], all row-major
-// float16, for gfx950 (MFMA v_mfma_f32_32x32x16_f16).
+// 16-bit x 16-bit -> fp32-accumulate GEMM, C[M,N] = A[M,K] * B[K,N], all row-major
+// float16 (or bfloat16 with DECA_BF16), for gfx950 (MFMA v_mfma_f32_32x32x16_f16 /
+// _bf16).
 //
 // One code object per (shape, GemmConfig); every DECA_* macro is a compile-time
 // constant supplied by kernels/gemm_hip.py, as the reference bakes shape and
@@ -29,6 +30,9 @@
 
 #ifndef DECA_BM
 #error "gemm.hip is a template: define the DECA_* macros"
+#endif
+#ifndef DECA_BF16
+#define DECA_BF16 0
 #endif
 
 #define M_ DECA_M
@@ -74,8 +78,15 @@ static_assert(GM % DECA_RASTER == 0, "raster group must divide the workgroup row
 static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
 static_assert(CPR_B >= 8, "BN >= 64");
 
-typedef _Float16 half8 __attribute__((ext_vector_type(8)));
-typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+#if DECA_BF16
+typedef __bf16 elem_t;
+#define DECA_MFMA __builtin_amdgcn_mfma_f32_32x32x16_bf16
+#else
+typedef _Float16 elem_t;
+#define DECA_MFMA __builtin_amdgcn_mfma_f32_32x32x16_f16
+#endif
+typedef elem_t half8 __attribute__((ext_vector_type(8)));
+typedef elem_t half4 __attribute__((ext_vector_type(4)));
 typedef short short4v __attribute__((ext_vector_type(4)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
@@ -99,8 +110,8 @@ __device__ __forceinline__ int b_chunk_slot(int k, int c) {
 }
 
 extern "C" __global__ void __launch_bounds__(NT)
-deca_main(const _Float16* __restrict__ A, const _Float16* __restrict__ B,
-          _Float16* __restrict__ C) {
+deca_main(const elem_t* __restrict__ A, const elem_t* __restrict__ B,
+          elem_t* __restrict__ C) {
   __shared__ __attribute__((aligned(16))) unsigned char lds[LDS_BYTES];
 
   const int tid = threadIdx.x;
@@ -125,8 +136,8 @@ deca_main(const _Float16* __restrict__ A, const _Float16* __restrict__ B,
   const int bm = (lin / GROUP) * DECA_RASTER + (lin % GROUP) % DECA_RASTER;
   const int bn = (lin % GROUP) / DECA_RASTER;
 
-  const _Float16* a_gbase = A + static_cast<size_t>(bm) * BM * K_;
-  const _Float16* b_gbase = B + static_cast<size_t>(bn) * BN;
+  const elem_t* a_gbase = A + static_cast<size_t>(bm) * BM * K_;
+  const elem_t* b_gbase = B + static_cast<size_t>(bn) * BN;
 
   // ---- accumulators and fragment addressing -----------------------------------
   floatx16 acc[MT][NTL];
@@ -175,7 +186,7 @@ deca_main(const _Float16* __restrict__ A, const _Float16* __restrict__ B,
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
       for (int nt = 0; nt < NTL; ++nt)
-        acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[nt], af[mt], acc[mt][nt], 0, 0, 0);
+        acc[mt][nt] = DECA_MFMA(bf[nt], af[mt], acc[mt][nt], 0, 0, 0);
   };
 
   // Scheduling pattern of one k-step: the LDS reads of the next fragments are
@@ -227,15 +238,15 @@ deca_main(const _Float16* __restrict__ A, const _Float16* __restrict__ B,
   // insertion does not see an LDS write and force vmcnt(0) before every LDS
   // read; the waits are explicit (DECA_WAIT_VMCNT) and paired with a barrier.
   // The "memory" clobber keeps LDS reads from moving across the issue point.
-  auto dma16 = [&](const _Float16* origin, unsigned voff, unsigned lds_addr) {
+  auto dma16 = [&](const elem_t* origin, unsigned voff, unsigned lds_addr) {
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                  :
                  : "v"(voff), "s"(origin), "s"(lds_addr)
                  : "memory");
   };
   auto issue_tile = [&](int kt, int slot) {
-    const _Float16* a_origin = a_gbase + kt * BK;
-    const _Float16* b_origin = b_gbase + static_cast<size_t>(kt) * BK * N_;
+    const elem_t* a_origin = a_gbase + kt * BK;
+    const elem_t* b_origin = b_gbase + static_cast<size_t>(kt) * BK * N_;
     const unsigned a_dst = lds_u + slot * A_STAGE_BYTES + wave_u * 1024;
     const unsigned b_dst = lds_u + STAGES * A_STAGE_BYTES + slot * B_STAGE_BYTES + wave_u * 1024;
 #pragma unroll
@@ -381,7 +392,7 @@ deca_main(const _Float16* __restrict__ A, const _Float16* __restrict__ B,
 #if DECA_EPI_LDS
   {
     constexpr int LD = BN + EPI_PAD;
-    _Float16* c_lds = reinterpret_cast<_Float16*>(lds);
+    elem_t* c_lds = reinterpret_cast<elem_t*>(lds);
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -390,7 +401,7 @@ deca_main(const _Float16* __restrict__ A, const _Float16* __restrict__ B,
         for (int q = 0; q < 4; ++q) {
           half4 h;
 #pragma unroll
-          for (int e = 0; e < 4; ++e) h[e] = static_cast<_Float16>(acc[mt][nt][q * 4 + e]);
+          for (int e = 0; e < 4; ++e) h[e] = static_cast<elem_t>(acc[mt][nt][q * 4 + e]);
           const int m = wm0 + mt * 32 + l32;
           const int n = wn0 + nt * 32 + q * 8 + khalf * 4;
           *reinterpret_cast<half4*>(c_lds + m * LD + n) = h;
@@ -398,7 +409,7 @@ deca_main(const _Float16* __restrict__ A, const _Float16* __restrict__ B,
     __syncthreads();
     constexpr int CPR_C = BN / 8;
     static_assert((BM * CPR_C) % NT == 0, "epilogue coverage");
-    _Float16* c_g = C + static_cast<size_t>(bm) * BM * N_ + static_cast<size_t>(bn) * BN;
+    elem_t* c_g = C + static_cast<size_t>(bm) * BM * N_ + static_cast<size_t>(bn) * BN;
 #pragma unroll
     for (int it = 0; it < BM * CPR_C / NT; ++it) {
       const int id = it * NT + tid;
@@ -409,7 +420,7 @@ deca_main(const _Float16* __restrict__ A, const _Float16* __restrict__ B,
   }
 #else
   {
-    _Float16* c_g = C + (static_cast<size_t>(bm) * BM + wm0 + l32) * N_ +
+    elem_t* c_g = C + (static_cast<size_t>(bm) * BM + wm0 + l32) * N_ +
                     static_cast<size_t>(bn) * BN + wn0 + khalf * 4;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
@@ -419,7 +430,7 @@ deca_main(const _Float16* __restrict__ A, const _Float16* __restrict__ B,
         for (int q = 0; q < 4; ++q) {
           half4 h;
 #pragma unroll
-          for (int e = 0; e < 4; ++e) h[e] = static_cast<_Float16>(acc[mt][nt][q * 4 + e]);
+          for (int e = 0; e < 4; ++e) h[e] = static_cast<elem_t>(acc[mt][nt][q * 4 + e]);
           *reinterpret_cast<half4*>(c_g + static_cast<size_t>(mt) * 32 * N_ + nt * 32 + q * 8) = h;
         }
   }

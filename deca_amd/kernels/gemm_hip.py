@@ -116,21 +116,26 @@ def check_config(cfg: GemmConfig, M: int, N: int, K: int, max_smem: int = MAX_LD
     assert est_regs_per_thread(cfg) <= MAX_VGPRS
 
 
-def make_gemm_tc(M: int, N: int, K: int, cfg: GemmConfig) -> KernelSpec:
+DTYPES = ("float16", "bfloat16")
+
+
+def make_gemm_tc(M: int, N: int, K: int, cfg: GemmConfig, dtype: str = "float16") -> KernelSpec:
     """Specialised kernel: 1-D grid of (M/BM)*(N/BN) workgroups of `threads`
-    lanes (reference: gemm_tir.py:156), static LDS."""
+    lanes (reference: gemm_tir.py:156), static LDS.  `dtype` is the type of A, B
+    and C (the reference is fp16 only; bf16 uses the bf16 MFMA of the same shape)."""
     check_config(cfg, M, N, K)
+    assert dtype in DTYPES
     defines = {
         "DECA_M": M, "DECA_N": N, "DECA_K": K,
         "DECA_BM": cfg.BM, "DECA_BN": cfg.BN, "DECA_BK": cfg.BK,
         "DECA_WM": cfg.warp_m, "DECA_WN": cfg.warp_n,
         "DECA_STAGES": cfg.stages, "DECA_RASTER": cfg.raster,
         "DECA_EPI_LDS": int(cfg.epi_smem), "DECA_XCD": int(cfg.xcd),
-        "DECA_DIRECT": int(cfg.direct),
+        "DECA_DIRECT": int(cfg.direct), "DECA_BF16": int(dtype == "bfloat16"),
     }
     return make_spec(
         TEMPLATE, defines, grid=((M // cfg.BM) * (N // cfg.BN), 1, 1), block=(cfg.threads, 1, 1),
-        nargs=3, options=FAST_MATH_OPTIONS, meta={"cfg": str(cfg)},
+        nargs=3, options=FAST_MATH_OPTIONS, meta={"cfg": str(cfg), "dtype": dtype},
     )
 
 
@@ -152,7 +157,8 @@ def build_gemm_tc(spec: KernelSpec, target: str | None = None, dump_dir: str | N
     return load_kernel(spec, path)
 
 
-def build_gemm_tc_to_file(shape, cfg: GemmConfig, arch: str, path: str) -> str:
+def build_gemm_tc_to_file(shape, cfg: GemmConfig, arch: str, path: str,
+                          dtype: str = "float16") -> str:
     """Builds in a worker process (no GPU context needed) and writes a code object."""
     M, N, K = shape
-    return build_kernel(make_gemm_tc(M, N, K, cfg), arch, path)
+    return build_kernel(make_gemm_tc(M, N, K, cfg, dtype), arch, path)

@@ -1,5 +1,6 @@
 """
-FP16 MFMA GEMM operator: C = A @ B with fp32 accumulation and fp16 output.
+16-bit MFMA GEMM operator: C = A @ B with fp32 accumulation; fp16 (the
+reference's type) or bf16 inputs and output.
 
 A `GemmConfig` fully determines a specialisation of `csrc/gemm.hip`
 (reference: src/operators/GEMMTC.py).
@@ -19,7 +20,9 @@ class GEMMTC(Operator):
         """`acc` must be "fp32": the matrix cores of CDNA4 have no fp16
         accumulation, so the reference's acc="fp16" / acc_splits modes
         (GEMMTC.py:29-43) do not exist here."""
-        assert dtype == "float16", "GEMMTC only supports float16 inputs"
+        from deca_amd.kernels.rowwise_bench import canonical_dtype
+
+        dtype = canonical_dtype(dtype)  # "float16" (the reference's only type) or "bfloat16"
         if acc != "fp32" or acc_splits != 1:
             raise NotImplementedError("MFMA accumulates in fp32 only")
         super().__init__(name)
@@ -33,14 +36,15 @@ class GEMMTC(Operator):
     def tolerance(self):
         """(atol, rtol) against the fp32 product: the fp16 output rounding is
         ~5e-4 relative and the accumulation error grows like sqrt(K)
-        (reference: GEMMTC.py:51-63)."""
-        return (1e-2 * math.sqrt(self.K / 1024), 2e-3)
+        (reference: GEMMTC.py:51-63); bf16 has 3 fewer mantissa bits (x8)."""
+        scale = 8.0 if self.dtype == "bfloat16" else 1.0
+        return (1e-2 * math.sqrt(self.K / 1024) * scale, 2e-3 * scale)
 
     def _check(self, cfg):
         gemm_hip.check_config(cfg, self.M, self.N, self.K)
 
     def _specialise(self, cfg):
-        return gemm_hip.make_gemm_tc(self.M, self.N, self.K, cfg)
+        return gemm_hip.make_gemm_tc(self.M, self.N, self.K, cfg, self.dtype)
 
     def _load(self, spec):
         return gemm_hip.build_gemm_tc(spec)
@@ -48,12 +52,14 @@ class GEMMTC(Operator):
     def make_inputs(self):
         from deca_amd.kernels.gemm_bench import make_inputs
 
-        return make_inputs(self.M, self.N, self.K)
+        from deca_amd.kernels.rowwise_bench import torch_dtype
+
+        return make_inputs(self.M, self.N, self.K, dtype=torch_dtype(self.dtype))
 
     def make_output(self, inputs):
         import torch
 
-        return torch.empty(self.M, self.N, device=inputs[0].device, dtype=torch.float16)
+        return torch.empty(self.M, self.N, device=inputs[0].device, dtype=inputs[0].dtype)
 
     def reference(self, inputs):
         """fp32 product of the fp16 inputs, with TF32-style shortcuts off: torch's

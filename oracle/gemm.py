@@ -39,6 +39,14 @@ def gemm_f16_out(a: np.ndarray, b: np.ndarray) -> np.ndarray:
         return gemm_f32(a, b).astype(np.float16).astype(np.float32)
 
 
+def gemm_bf16_out(a: np.ndarray, b: np.ndarray) -> np.ndarray:
+    """The bf16 variant (no counterpart in the reference, which is fp16 only):
+    same fp32 accumulation, one round-to-nearest-even conversion to bf16."""
+    from oracle.rowwise import round_to_dtype
+
+    return round_to_dtype(gemm_f32(a, b), "bfloat16")
+
+
 def gemm_loops(a: np.ndarray, b: np.ndarray) -> np.ndarray:
     """Triple loop in fp32, k ascending (small sizes only)."""
     a = np.asarray(a, np.float32)

@@ -30,6 +30,8 @@ def parse_args(argv=None):
                         metavar=("M", "N", "K"))
     parser.add_argument("--sweep", action="store_true", default=False,
                         help="tune the square 2K-16K benchmark grid")
+    parser.add_argument("--dtype", choices=["fp16", "bf16"], default="fp16",
+                        help="type of A, B and C (accumulation is always fp32)")
     parser.add_argument("--top_n", type=int, default=24,
                         help="number of ranked configs to compile and measure (0 = all)")
     parser.add_argument("--jobs", type=int, default=min(16, os.cpu_count() or 1),
@@ -45,7 +47,7 @@ def tune(args, shape, arch, arch_str, log):
     from deca_amd.Tuner import Tuner
 
     tuner = Tuner("GEMM", arch, arch_str, args.top_n, args.jobs, args.finalists, args.rounds)
-    return tuner.tune(*shape, log=log)
+    return tuner.tune(*shape, log=log, dtype=args.dtype)
 
 
 def write_sweep_csv(summary, path):

@@ -83,8 +83,17 @@ GEMM_FULL = [
 ]
 
 
+# bf16 inputs / output (fp32 accumulate)
+GEMM_BF16_CASES = [
+    (512, 512, 512, GemmConfig(256, 256, 64, 128, 64, 2, 1, False, False, True)),
+    (512, 1024, 256, GemmConfig(128, 128, 32, 64, 64, 3, 2, True, True, True)),
+    (256, 256, 192, GemmConfig(64, 64, 64, 32, 32, 1, 1, False, False, False)),
+]
+
+
 def gemm_specs():
-    return [make_gemm_tc(M, N, K, cfg) for M, N, K, cfg in GEMM_CASES + GEMM_FULL]
+    return ([make_gemm_tc(M, N, K, cfg) for M, N, K, cfg in GEMM_CASES + GEMM_FULL] +
+            [make_gemm_tc(M, N, K, cfg, "bfloat16") for M, N, K, cfg in GEMM_BF16_CASES])
 
 
 # (B, H, S_q, S_kv, D, causal, cfg): sizes the CPU checker finishes in seconds

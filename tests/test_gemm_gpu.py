@@ -13,7 +13,7 @@ import numpy as np
 import pytest
 import torch
 
-from kernel_cases import GEMM_CASES, GEMM_FULL
+from kernel_cases import GEMM_BF16_CASES, GEMM_CASES, GEMM_FULL
 from oracle import gemm as og
 
 pytestmark = pytest.mark.gpu
@@ -123,3 +123,31 @@ def test_gemm_full_size(M, N, K, cfg):
         worst = max(worst, (c[r0:r0 + 1024].float() - ref).abs().max().item())
         scale = max(scale, ref.abs().max().item())
     assert worst / scale <= REL_GATE
+
+
+@pytest.mark.parametrize("M,N,K,cfg", GEMM_BF16_CASES, ids=lambda v: str(v))
+def test_gemm_bf16_parity(M, N, K, cfg):
+    """bf16 inputs and output, fp32 accumulation: same gate (max rel err <= 1e-2
+    against the fp32 product), and at most one bf16 ulp from the checker."""
+    from deca_amd.kernels.gemm_bench import make_inputs_cpu
+    from deca_amd.kernels.gemm_hip import build_gemm_tc, make_gemm_tc
+
+    print(f"case gemm bf16 {M}x{N}x{K} {cfg}", flush=True)
+    a, b = make_inputs_cpu(M, N, K, seed=K, dtype=torch.bfloat16)
+    kern = build_gemm_tc(make_gemm_tc(M, N, K, cfg, "bfloat16"))
+    c = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    kern(a.cuda(), b.cuda(), c)
+    torch.cuda.synchronize()
+    got = c.float().cpu().numpy()
+    af, bf = a.float().numpy(), b.float().numpy()
+    ref = og.gemm_f32(af, bf)
+    assert np.isfinite(got).all()
+    assert og.max_rel_err(got, ref) <= REL_GATE
+    want = og.gemm_bf16_out(af, bf)
+    assert np.all(np.abs(got - want) <= np.maximum(np.abs(want), 2.0**-14) * 2.0**-7 * 1.001 + 1e-3)
+    assert (got != want).mean() < 0.05
+    # identity: A @ I == A exactly
+    eye = torch.eye(K, N).bfloat16()
+    kern(a.cuda(), eye.cuda(), c)
+    torch.cuda.synchronize()
+    assert torch.equal(c.cpu()[:, :min(K, N)], a[:, :min(K, N)])

@@ -60,3 +60,9 @@ def test_error_metrics():
     assert atol == 1e-2 and rtol == 2e-3
     assert abs(og.excess(c, ref, 1024) - 0.004 / (1e-2 + 2e-3 * 4)) < 1e-4
     assert og.gemm_flops(8192, 8192, 8192) == 2.0 * 8192**3
+
+
+def test_bf16_output_rounding():
+    a, b = _rand(16, 64, 4), _rand(64, 16, 5)
+    want = torch.from_numpy(og.gemm_f32(a, b)).bfloat16().float().numpy()
+    assert np.array_equal(og.gemm_bf16_out(a, b), want)
