@@ -28,32 +28,19 @@ MFMA_PEAK_TFLOPS = 2500.0
 MALL_BYTES = 256 * 1024 * 1024
 
 
-def _tuned():
-    with open(os.path.join(ROOT, "deca_amd", "tuned_configs.json")) as f:
-        return json.load(f)
+def _cfg(operator, shape, dtype="float16", causal=False):
+    """The stored winner of a tuning run for this workload."""
+    from deca_amd import tuned
 
-
-def _row_cfg(d):
-    from deca_amd.kernels.rowwise_hip import RowConfig
-
-    return RowConfig(**d)
-
-
-def _gemm_cfg(d):
-    from deca_amd.kernels.gemm_hip import GemmConfig
-
-    return GemmConfig(**d)
-
-
-def _fa_cfg(d):
-    from deca_amd.kernels.flash_attn_hip import FAConfig
-
-    return FAConfig(**d)
+    key = tuned.make_key(operator, shape, dtype, "gfx950", causal)
+    cfg = tuned.lookup(key)
+    if cfg is None:
+        raise KeyError(f"no tuned config for {key}: run the matching test_*.py driver with --cache")
+    return cfg
 
 
 # name -> description of the workload (the benchmark configurations)
 def workloads():
-    t = _tuned()
     w = {}
     for name, (op, M, N, dtype) in {
         "rmsnorm_bf16_16384x4096": ("rmsnorm", 16384, 4096, "bfloat16"),
@@ -61,15 +48,14 @@ def workloads():
         "rmsnorm_fp16_8192x8192": ("rmsnorm", 8192, 8192, "float16"),
     }.items():
         w[name] = {"kind": "rowwise", "op": op, "M": M, "N": N, "dtype": dtype,
-                   "cfg": _row_cfg(t[name])}
+                   "cfg": _cfg(op, (M, N), dtype)}
     for n in (2048, 4096, 8192, 12288, 16384):
-        name = f"gemm_fp16_{n}"
-        w[name] = {"kind": "gemm", "M": n, "N": n, "K": n, "cfg": _gemm_cfg(t[name])}
+        w[f"gemm_fp16_{n}"] = {"kind": "gemm", "M": n, "N": n, "K": n, "cfg": _cfg("GEMM", (n, n, n))}
     for D in (128, 64):
         for causal in (False, True):
             name = f"fa_fp16_b4h16s4096d{D}" + ("_causal" if causal else "")
             w[name] = {"kind": "fa", "B": 4, "H": 16, "S": 4096, "D": D, "causal": causal,
-                       "cfg": _fa_cfg(t[name])}
+                       "cfg": _cfg("flash_attn", (4, 16, 4096, 4096, D), "float16", causal)}
     for k, v in w.items():
         v["name"] = k
     return w

@@ -77,7 +77,7 @@ class Tuner:
 
     def __init__(self, operator: str = "GEMM", arch=None, arch_str: str | None = None,
                  top_n: int | None = None, jobs: int | None = None, finalists: int = 3,
-                 rounds: int = 5):
+                 rounds: int = 5, cache_path: str | None = None):
         assert operator in self.OPERATORS
         self.operator = operator
         if arch is None:
@@ -90,6 +90,8 @@ class Tuner:
         self.jobs = jobs if jobs is not None else min(16, os.cpu_count() or 1)
         self.finalists = finalists
         self.rounds = rounds
+        # JSON file of stored winners (see deca_amd/tuned.py); None: always search
+        self.cache_path = cache_path
 
     # -- the three compute levels of the reference's stub map onto the stages ----
     def tune_cpt_0(self, *shape, **kw):
@@ -197,11 +199,21 @@ class Tuner:
         from deca_amd.kernels.attn_bench import bench_interleaved
         from deca_amd.RuntimeMod import RuntimeMod
 
+        from deca_amd import tuned
+
         start = time.time()
         op = self._make_op(shape, **kw)
-        configs = self._solve(op, shape, **kw)
-        ranked = self._rank(configs, shape, **kw)
-        print(f"Find {len(configs)} {op.name} configs, measuring {len(ranked)}", flush=True)
+        key = tuned.make_key(self.operator, getattr(op, "shape", shape), op.dtype, self.arch_str,
+                             bool(getattr(op, "causal", False)))
+        cached = tuned.lookup(key, self.cache_path) if self.cache_path else None
+        if cached is not None and op.is_valid(cached):
+            # a stored winner: verify and time it alone instead of searching
+            configs = ranked = [cached]
+            print(f"Using the stored {op.name} config of {key}", flush=True)
+        else:
+            configs = self._solve(op, shape, **kw)
+            ranked = self._rank(configs, shape, **kw)
+            print(f"Find {len(configs)} {op.name} configs, measuring {len(ranked)}", flush=True)
 
         fn_path, args_for = self._builder(op, shape)
         paths = build_all(fn_path, {cfg: args_for(cfg) for cfg in ranked}, self.jobs)
@@ -257,6 +269,11 @@ class Tuner:
         if log is not None:
             log.write(msg + "\n")
             log.flush()
+        if self.cache_path:
+            unit = "GB/s" if self.operator in ("softmax", "rmsnorm") else "TFLOPS"
+            tuned.store(key, best_cfg, best, unit, self.cache_path, runtime_ms=round(best_t * 1e3, 4),
+                        max_err=float(f"{err_of[best_cfg]:.3e}"), measured_on=self.arch.name,
+                        candidates=len(ranked))
         for kern in keep:
             kern.close()
         return best_cfg, best, ref

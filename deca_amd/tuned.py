@@ -1,0 +1,66 @@
+"""Persisted best configurations, keyed by operator / shape / dtype / architecture.
+
+The reference re-tunes on every run (its compiled kernels live in a temporary
+directory, test_gemm_tc.py:74).  Here the winner of a tuning run can be stored
+in a JSON file and looked up later, so that repeated runs -- and bench.py --
+skip the search.  The file shipped with the package holds the winners measured
+on an MI355X for the benchmark configurations.
+"""
+
+from __future__ import annotations
+
+import json
+import os
+
+DEFAULT_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "tuned_configs.json")
+
+
+def make_key(operator: str, shape, dtype: str = "float16", arch: str = "gfx950",
+             causal: bool = False) -> str:
+    dims = "x".join(str(int(d)) for d in shape)
+    return f"{operator}|{dims}|{dtype}{'|causal' if causal else ''}|{arch}"
+
+
+def _config_class(operator: str):
+    if operator == "GEMM":
+        from deca_amd.kernels.gemm_hip import GemmConfig
+
+        return GemmConfig
+    if operator in ("softmax", "rmsnorm"):
+        from deca_amd.kernels.rowwise_hip import RowConfig
+
+        return RowConfig
+    if operator == "flash_attn":
+        from deca_amd.kernels.flash_attn_hip import FAConfig
+
+        return FAConfig
+    raise KeyError(operator)
+
+
+def load(path: str | None = None) -> dict:
+    path = path or DEFAULT_PATH
+    if not os.path.exists(path):
+        return {}
+    with open(path) as f:
+        return json.load(f)
+
+
+def lookup(key: str, path: str | None = None):
+    """The stored config object of `key`, or None."""
+    entry = load(path).get(key)
+    if entry is None:
+        return None
+    return _config_class(key.split("|")[0])(**entry["config"])
+
+
+def store(key: str, cfg, throughput: float, unit: str, path: str | None = None, **extra) -> None:
+    """Records `cfg` as the winner of `key` (atomic rewrite of the JSON file)."""
+    path = path or DEFAULT_PATH
+    table = load(path)
+    table[key] = {"config": cfg.as_dict(), "throughput": round(float(throughput), 2), "unit": unit,
+                  **extra}
+    tmp = f"{path}.tmp{os.getpid()}"
+    with open(tmp, "w") as f:
+        json.dump(table, f, indent=1, sort_keys=True)
+        f.write("\n")
+    os.replace(tmp, path)

@@ -38,15 +38,27 @@ def parse_args(argv=None):
                         help="parallel compile workers")
     parser.add_argument("--finalists", type=int, default=3,
                         help="best configs re-timed against torch in the final round")
+    parser.add_argument("--cache", nargs="?", const="", default=None, metavar="JSON",
+                        help="store the winner in (and reuse it from) a JSON file; without a "
+                             "path, the table shipped with the package")
     parser.add_argument("--rounds", type=int, default=5,
                         help="interleaved timing rounds of the final comparison")
     return parser.parse_args(argv)
 
 
+def _cache_path(args):
+    if args.cache is None:
+        return None
+    from deca_amd import tuned
+
+    return args.cache or tuned.DEFAULT_PATH
+
+
 def tune(args, shape, arch, arch_str, log):
     from deca_amd.Tuner import Tuner
 
-    tuner = Tuner("GEMM", arch, arch_str, args.top_n, args.jobs, args.finalists, args.rounds)
+    tuner = Tuner("GEMM", arch, arch_str, args.top_n, args.jobs, args.finalists, args.rounds,
+                  cache_path=_cache_path(args))
     return tuner.tune(*shape, log=log, dtype=args.dtype)
 
 

@@ -181,3 +181,28 @@ def test_runtime_mod_error_metric_and_nan():
     with pytest.raises(RuntimeError, match="no kernel loaded"):
         rt.time_kernel_op()
     assert rt.is_flash_attn is False
+
+
+def test_tuned_table_roundtrip(tmp_path):
+    from deca_amd import tuned
+    from deca_amd.kernels.flash_attn_hip import FAConfig
+    from deca_amd.kernels.gemm_hip import GemmConfig
+
+    path = str(tmp_path / "t.json")
+    assert tuned.lookup("softmax|16384x4096|float16|gfx950", path) is None
+    k1 = tuned.make_key("softmax", (16384, 4096), "float16")
+    k2 = tuned.make_key("flash_attn", (4, 16, 4096, 4096, 128), "float16", "gfx950", causal=True)
+    k3 = tuned.make_key("GEMM", (8192, 8192, 8192), "bfloat16")
+    assert k1 == "softmax|16384x4096|float16|gfx950"
+    assert k2 == "flash_attn|4x16x4096x4096x128|float16|causal|gfx950"
+    tuned.store(k1, RowConfig(256, 2, 8, hint=True), 6391.3, "GB/s", path, runtime_ms=0.042)
+    tuned.store(k2, FAConfig(256, 128, 8, 2), 800.0, "TFLOPS", path)
+    tuned.store(k3, GemmConfig(256, 256, 64, 128, 64, 2, 4), 1200.0, "TFLOPS", path)
+    assert tuned.lookup(k1, path) == RowConfig(256, 2, 8, hint=True)
+    assert tuned.lookup(k2, path) == FAConfig(256, 128, 8, 2)
+    assert tuned.lookup(k3, path) == GemmConfig(256, 256, 64, 128, 64, 2, 4)
+    assert tuned.load(path)[k1]["runtime_ms"] == 0.042
+    # the table shipped with the package covers every bench workload
+    import bench
+
+    assert len(bench.workloads()) == 12
