@@ -129,7 +129,14 @@ class RuntimeMod:
                         f"{self.compute_pattern}: max error {self.max_error:.3e} exceeds "
                         f"atol={atol} + rtol={rtol} * |ref| (x{excess:.2f})")
             del ref
-        self.execution_time = t = bench_cuda(lambda: kern(*args))
+        if getattr(op, "metric", "GB/s") == "GB/s":
+            # memory-bound: cycle through buffer sets larger than the Infinity Cache
+            from deca_amd.kernels.rowwise_bench import cycle, rotating_sets
+
+            sets = rotating_sets(inputs, args[-1], getattr(self.arch, "mall_bytes", 0))
+            self.execution_time = t = bench_cuda(cycle(kern, sets))
+        else:
+            self.execution_time = t = bench_cuda(lambda: kern(*args))
         return t
 
     # ---- timing ----------------------------------------------------------------------------

@@ -349,6 +349,7 @@ FA_DOMAINS = {
     "bc": (32, 64, 128),
     "nw": (1, 2, 4, 8),
     "st": (1, 2),
+    "pipe": (0, 1),
 }
 
 
@@ -358,7 +359,7 @@ def _fa_constraints(arch, B: int, H: int, S_q: int, S_kv: int, D: int, type_size
     simds = arch.simds_per_cu
 
     def build(o, v):
-        br, bc, nw, st = (v[k] for k in FA_DOMAINS)
+        br, bc, nw, st, pipe = (v[k] for k in FA_DOMAINS)
         c = o.const
         threads = nw * wave
         cpr = D // 8
@@ -375,12 +376,14 @@ def _fa_constraints(arch, B: int, H: int, S_q: int, S_kv: int, D: int, type_size
             o.ule(threads, c(arch.max_threads_per_block)),
             # LDS: `st` K tiles and `st` V tiles
             o.ule(st * bc * (2 * D * type_size), c(arch.max_dyn_smem_per_block)),
+            # the software-pipelined loop runs one K tile ahead: two slots, two tiles
+            o.implies(o.eq(pipe, c(1)), o.all_of(o.eq(st, c(2)), o.uge(o.udiv(c(S_kv), bc), c(2)))),
         ]
         # registers: O^T accumulator + S^T accumulator + P + Q fragments + K/V fragments
         mq = o.udiv(br, nw * 32)
         o_acc = mq * (D // 32 * 16)
-        s_acc = mq * o.udiv(bc, c(2))
         p_h = mq * o.udiv(bc, c(4))
+        s_acc = mq * o.udiv(bc, c(2)) * (pipe + 1)  # the pipelined loop keeps two S^T tiles
         q_frag = mq * (D // 16 * 4)
         regs = o_acc + s_acc + p_h + q_frag + 16 + mq * 4 + 40
         regs8 = o.udiv(regs + 7, c(8)) * 8
@@ -409,5 +412,5 @@ def solve_flash_attn(arch, B: int, H: int, S_q: int, S_kv: int, D: int, type_siz
     from deca_amd.kernels.flash_attn_hip import FAConfig
 
     cons = _fa_constraints(arch, B, H, S_q, S_kv, D, type_size, max_est_regs)
-    return [FAConfig(Br=br, Bc=bc, num_warps=nw, stages=st)
-            for br, bc, nw, st in _enumerate(FA_DOMAINS, cons, count, backend)]
+    return [FAConfig(Br=br, Bc=bc, num_warps=nw, stages=st, pipe=bool(pipe))
+            for br, bc, nw, st, pipe in _enumerate(FA_DOMAINS, cons, count, backend)]

@@ -77,7 +77,7 @@ class Tuner:
 
     def __init__(self, operator: str = "GEMM", arch=None, arch_str: str | None = None,
                  top_n: int | None = None, jobs: int | None = None, finalists: int = 3,
-                 rounds: int = 5, cache_path: str | None = None):
+                 rounds: int = 5, cache_path: str | None = None, retune: bool = False):
         assert operator in self.OPERATORS
         self.operator = operator
         if arch is None:
@@ -92,6 +92,7 @@ class Tuner:
         self.rounds = rounds
         # JSON file of stored winners (see deca_amd/tuned.py); None: always search
         self.cache_path = cache_path
+        self.retune = retune  # search even when a winner is stored (and replace it)
 
     # -- the three compute levels of the reference's stub map onto the stages ----
     def tune_cpt_0(self, *shape, **kw):
@@ -205,7 +206,7 @@ class Tuner:
         op = self._make_op(shape, **kw)
         key = tuned.make_key(self.operator, getattr(op, "shape", shape), op.dtype, self.arch_str,
                              bool(getattr(op, "causal", False)))
-        cached = tuned.lookup(key, self.cache_path) if self.cache_path else None
+        cached = tuned.lookup(key, self.cache_path) if self.cache_path and not self.retune else None
         if cached is not None and op.is_valid(cached):
             # a stored winner: verify and time it alone instead of searching
             configs = ranked = [cached]
@@ -252,12 +253,24 @@ class Tuner:
         inputs = op.make_inputs()
         out = op.make_output(inputs) if hasattr(op, "make_output") else torch.empty_like(inputs[0])
         args = op.kernel_args(inputs, out)
-        fns = {"torch": self._torch_fn(op, inputs)}
         keep = []
-        for _, cfg, _, _ in finalists:
-            kern = load_kernel(op.build_mod(cfg), paths[cfg])
-            keep.append(kern)
-            fns[cfg] = lambda kern=kern: kern(*args)
+        if self.operator in ("softmax", "rmsnorm"):
+            # memory-bound: DeCA and torch both cycle through buffer sets larger
+            # than the Infinity Cache, so that both stream from HBM
+            from deca_amd.kernels.rowwise_bench import cycle, rotating_sets
+
+            sets = rotating_sets(inputs, out, getattr(self.arch, "mall_bytes", 0))
+            fns = {"torch": cycle(lambda *a: op.reference(a[:-1]), sets)}
+            for _, cfg, _, _ in finalists:
+                kern = load_kernel(op.build_mod(cfg), paths[cfg])
+                keep.append(kern)
+                fns[cfg] = cycle(kern, sets)
+        else:
+            fns = {"torch": self._torch_fn(op, inputs)}
+            for _, cfg, _, _ in finalists:
+                kern = load_kernel(op.build_mod(cfg), paths[cfg])
+                keep.append(kern)
+                fns[cfg] = lambda kern=kern: kern(*args)
         times = bench_interleaved(fns, rounds=self.rounds)
         torch_t = times.pop("torch")
         best_cfg, best_t = min(times.items(), key=lambda x: x[1])

@@ -263,7 +263,9 @@ def fa_score(cfg, arch, shape, causal: bool = False) -> float:
     # vector-ALU time per FLOP: (4 + 4) lane-cycles per score element, 4 * D FLOPs each
     valu_rate = cus * arch.simds_per_cu * 16 * arch.sm_clock_hz  # lane-ops per second
     t_valu = (8.0 / (4.0 * D)) * cus / valu_rate
-    overlap = min(1.0, max(0.0, waves_per_simd - 1.0))  # share of VALU work hidden by other waves
+    # share of the VALU work hidden under matrix work: by other waves on the SIMD,
+    # or by the wave itself when its loop is software pipelined
+    overlap = min(1.0, max(0.0, waves_per_simd - 1.0) + (0.5 if cfg.pipe else 0.0))
     terms = sorted([t_mma, t_lds, t_l2])
     t_flop = terms[-1] + 0.3 * (terms[0] + terms[1]) + (1.0 - 0.8 * overlap) * t_valu
     t_flop = max(t_flop, t_valu)

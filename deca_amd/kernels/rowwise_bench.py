@@ -67,6 +67,35 @@ def make_inputs_cpu(op: str, M: int, N: int, dtype: str, seed: int = 0, std: flo
     return make_inputs(op, M, N, dtype, seed, "cpu", std)
 
 
+def rotating_sets(inputs, out, cache_bytes: int, factor: int = 4):
+    """Copies of (inputs..., out) whose total size is `factor` times the
+    last-level cache, to be cycled through while timing a memory-bound kernel.
+
+    The reference times every kernel on one set of buffers
+    (attn_bench.py:46-70).  On MI355X one [16384, 4096] fp16 input/output pair
+    is 268 MB next to a 256 MiB Infinity Cache, so a single set is partly served
+    from that cache and over-states the HBM rate; rotating sets larger than the
+    cache makes every launch stream from HBM."""
+    per_set = sum(t.numel() * t.element_size() for t in (*inputs, out))
+    n = max(1, -(-factor * cache_bytes // per_set))
+    sets = [(*inputs, out)]
+    for _ in range(n - 1):
+        sets.append((*(t.clone() for t in inputs), out.clone()))
+    return sets
+
+
+def cycle(fn, sets):
+    """A zero-argument callable that calls `fn(*sets[i])` with i advancing on every call."""
+    state = {"i": 0}
+
+    def call():
+        args = sets[state["i"] % len(sets)]
+        state["i"] += 1
+        return fn(*args)
+
+    return call
+
+
 def torch_ref(op: str, inputs, eps: float = RMSNORM_EPS):
     """Eager torch operator: the baseline and the correctness reference while tuning."""
     import torch

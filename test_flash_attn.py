@@ -39,6 +39,8 @@ def parse_args(argv=None):
     parser.add_argument("--cache", nargs="?", const="", default=None, metavar="JSON",
                         help="store the winner in (and reuse it from) a JSON file; without a "
                              "path, the table shipped with the package")
+    parser.add_argument("--retune", action="store_true", default=False,
+                        help="with --cache: search again and replace the stored winner")
     parser.add_argument("--rounds", type=int, default=5,
                         help="interleaved timing rounds of the final comparison")
     return parser.parse_args(argv)
@@ -64,7 +66,7 @@ def tune(args, shape, arch, arch_str, log):
     from deca_amd.Tuner import Tuner
 
     tuner = Tuner("flash_attn", arch, arch_str, args.top_n, args.jobs, args.finalists, args.rounds,
-                  cache_path=_cache_path(args))
+                  cache_path=_cache_path(args), retune=args.retune)
     return tuner.tune(*shape, log=log, causal=args.causal)
 
 

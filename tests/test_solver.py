@@ -119,13 +119,14 @@ def test_flash_attn_configs_are_valid(D, S):
         fa.check_config(cfg, S, S, D)
         assert (S // cfg.Br) * B * H >= ARCH.sm_nums
     want = set()
-    for br, bc, nw, st in itertools.product((32, 64, 128, 256), (32, 64, 128), (1, 2, 4, 8), (1, 2)):
-        cfg = fa.FAConfig(br, bc, nw, st)
+    for br, bc, nw, st, pipe in itertools.product((32, 64, 128, 256), (32, 64, 128), (1, 2, 4, 8),
+                                                   (1, 2), (False, True)):
+        cfg = fa.FAConfig(br, bc, nw, st, pipe=pipe)
         try:
             fa.check_config(cfg, S, S, D)
         except AssertionError:
             continue
-        if (S // br) * B * H < ARCH.sm_nums or st > S // bc:
+        if (S // br) * B * H < ARCH.sm_nums or st > S // bc or (pipe and S // bc < 2):
             continue
         regs = (fa.est_regs_per_thread(cfg, D) + 7) // 8 * 8
         if regs * -(-nw // 4) > 512:

@@ -206,3 +206,21 @@ def test_tuned_table_roundtrip(tmp_path):
     import bench
 
     assert len(bench.workloads()) == 12
+
+
+def test_rotating_sets_and_cycle():
+    import torch
+
+    from deca_amd.kernels.rowwise_bench import cycle, rotating_sets
+
+    x, w, y = torch.ones(64, 32), torch.ones(32), torch.zeros(64, 32)
+    per_set = (64 * 32 * 2 + 32) * 4
+    sets = rotating_sets((x, w), y, cache_bytes=per_set, factor=4)
+    assert len(sets) == 4 and sets[0][0] is x and sets[1][0] is not x
+    assert all(torch.equal(s[0], x) and len(s) == 3 for s in sets)
+    assert len(rotating_sets((x,), y, cache_bytes=0)) == 1
+    seen = []
+    call = cycle(lambda *a: seen.append(a[-1].data_ptr()), sets)
+    for _ in range(6):
+        call()
+    assert seen[:4] == [s[-1].data_ptr() for s in sets] and seen[4:] == seen[:2]
