@@ -227,11 +227,23 @@ def run_fa(wl, steps, warmup, with_cpu):
     return res
 
 
+def _measured_traffic(name):
+    """HBM-side bytes per launch measured with rocprofv3 counters (see
+    deca_amd/measured_traffic.json and profiles/), or None when not recorded."""
+    path = os.path.join(ROOT, "deca_amd", "measured_traffic.json")
+    if not os.path.exists(path):
+        return None
+    with open(path) as f:
+        entry = json.load(f).get("workloads", {}).get(name)
+    return entry["traffic_bytes"] if entry else None
+
+
 def run(wl, steps, warmup, with_cpu=True):
     t0 = time.perf_counter()
     print(f"[bench] {wl['name']} ...", file=sys.stderr, flush=True)
     res = {"rowwise": run_rowwise, "gemm": run_gemm, "fa": run_fa}[wl["kind"]](
         wl, steps, warmup, with_cpu)
+    res["roofline"]["traffic"] = _measured_traffic(wl["name"])
     print(f"[bench] {wl['name']}: {res['value']:.1f} {res['unit']} "
           f"({100 * res['roofline']['frac']:.1f}% of peak) in {time.perf_counter() - t0:.1f} s",
           file=sys.stderr, flush=True)
