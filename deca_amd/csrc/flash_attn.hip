@@ -45,6 +45,9 @@
 #define BC DECA_BC
 #define NW DECA_NW
 #define STAGES DECA_STAGES
+#ifndef DECA_EPI_LDS
+#define DECA_EPI_LDS 1
+#endif
 
 constexpr int NT = NW * 64;
 constexpr int WQ = BR / NW;       // query rows per wave
@@ -507,12 +510,24 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
 #endif
 
   // ---- epilogue: O[q][d] = O^T[d][q] / l ----------------------------------------------
-  // o_acc[dt][mq][e]: q = mq*32 + lane%32, d = dt*32 + (e/4)*8 + half*4 + e%4
+  // o_acc[dt][mq][e]: q = mq*32 + lane%32, d = dt*32 + (e/4)*8 + half*4 + e%4.
+  // A lane owns 8-byte pieces of a row; when the K/V ring is large enough the
+  // wave's [WQ][D] tile is staged through it (rows padded by 8 halves to spread
+  // the banks) and written with 16-byte stores that cover whole rows.
+  constexpr int EPI_LD = D_ + 8;
+  constexpr bool EPI_LDS = DECA_EPI_LDS && LDS_BYTES >= BR * EPI_LD * 2;
+  typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+  if (EPI_LDS) {
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+    __builtin_amdgcn_s_barrier();  // every wave is done reading K/V tiles
+  }
+  _Float16* o_lds = reinterpret_cast<_Float16*>(lds) + wave * WQ * EPI_LD;
 #pragma unroll
   for (int mq = 0; mq < MQ; ++mq) {
     const float l = l_i[mq] + __shfl_xor(l_i[mq], 32, 64);
     const float inv = 1.0f / l;
-    _Float16* o_row = o_base + (mq * 32 + l32) * D_ + half * 4;
+    _Float16* o_row = EPI_LDS ? o_lds + (mq * 32 + l32) * EPI_LD + half * 4
+                              : o_base + (mq * 32 + l32) * D_ + half * 4;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -522,5 +537,18 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
         for (int e = 0; e < 4; ++e) h[e] = static_cast<_Float16>(o_acc[dt][mq][g * 4 + e] * inv);
         *reinterpret_cast<half4*>(o_row + dt * 32 + g * 8) = h;
       }
+  }
+  if (EPI_LDS) {
+    // the tile is private to the wave: its own LDS writes only need to have landed
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+    __builtin_amdgcn_wave_barrier();
+    constexpr int CHUNKS = WQ * CPR;  // 16-byte chunks of the wave's tile
+#pragma unroll
+    for (int it = 0; it < CHUNKS / 64; ++it) {
+      const int idx = it * 64 + lane;
+      const int row = idx / CPR, c = idx % CPR;
+      const u32x4 v = *reinterpret_cast<const u32x4*>(o_lds + row * EPI_LD + c * 8);
+      *reinterpret_cast<u32x4*>(o_base + row * D_ + c * 8) = v;
+    }
   }
 }
