@@ -349,18 +349,21 @@ FA_DOMAINS = {
     "bc": (32, 64, 128),
     "nw": (1, 2, 4, 8),
     "st": (1, 2),
-    "pipe": (0, 1),
+    "pipe": (0, 1, 2),
 }
 
 
 def _fa_constraints(arch, B: int, H: int, S_q: int, S_kv: int, D: int, type_size: int,
                     max_est_regs: int):
+    from deca_amd.kernels.flash_attn_hip import slot_schedule_ok
+
     wave = arch.warp_size
     simds = arch.simds_per_cu
 
     def build(o, v):
         br, bc, nw, st, pipe = (v[k] for k in FA_DOMAINS)
         c = o.const
+        slot_bcs = [b for b in FA_DOMAINS["bc"] if slot_schedule_ok(b, D)] or [0]
         threads = nw * wave
         cpr = D // 8
         out = [
@@ -377,13 +380,16 @@ def _fa_constraints(arch, B: int, H: int, S_q: int, S_kv: int, D: int, type_size
             # LDS: `st` K tiles and `st` V tiles
             o.ule(st * bc * (2 * D * type_size), c(arch.max_dyn_smem_per_block)),
             # the software-pipelined loop runs one K tile ahead: two slots, two tiles
-            o.implies(o.eq(pipe, c(1)), o.all_of(o.eq(st, c(2)), o.uge(o.udiv(c(S_kv), bc), c(2)))),
+            o.implies(o.uge(pipe, c(1)), o.all_of(o.eq(st, c(2)), o.uge(o.udiv(c(S_kv), bc), c(2)))),
+            # the slot-interleaved loop issues the S^T chains in pairs of 32-key blocks
+            o.implies(o.eq(pipe, c(2)), o.any_of(*[o.eq(bc, c(b)) for b in slot_bcs])),
         ]
         # registers: O^T accumulator + S^T accumulator + P + Q fragments + K/V fragments
         mq = o.udiv(br, nw * 32)
         o_acc = mq * (D // 32 * 16)
         p_h = mq * o.udiv(bc, c(4))
-        s_acc = mq * o.udiv(bc, c(2)) * (pipe + 1)  # the pipelined loop keeps two S^T tiles
+        # the pipelined loops keep two S^T tiles
+        s_acc = mq * o.udiv(bc, c(2)) * o.ite(o.uge(pipe, c(1)), c(2), c(1))
         q_frag = mq * (D // 16 * 4)
         regs = o_acc + s_acc + p_h + q_frag + 16 + mq * 4 + 40
         regs8 = o.udiv(regs + 7, c(8)) * 8
@@ -412,5 +418,5 @@ def solve_flash_attn(arch, B: int, H: int, S_q: int, S_kv: int, D: int, type_siz
     from deca_amd.kernels.flash_attn_hip import FAConfig
 
     cons = _fa_constraints(arch, B, H, S_q, S_kv, D, type_size, max_est_regs)
-    return [FAConfig(Br=br, Bc=bc, num_warps=nw, stages=st, pipe=bool(pipe))
+    return [FAConfig(Br=br, Bc=bc, num_warps=nw, stages=st, pipe=int(pipe))
             for br, bc, nw, st, pipe in _enumerate(FA_DOMAINS, cons, count, backend)]

@@ -13,6 +13,8 @@
 //   DECA_SCALE          softmax scale
 //   DECA_PIPE           1: S^T of the next tile is computed before the softmax of
 //                       the current one (two S^T accumulators per wave)
+//                       2: as 1, and every matrix instruction of an iteration carries
+//                       a fixed share of the iteration's vector work ("slots")
 //
 // The problem is computed transposed, which is what makes the two MFMA
 // products chain without a layout change on CDNA:
@@ -35,6 +37,8 @@
 // l = l * alpha + sum p (fp32 p); P = fp16(p) feeds the second product;
 // O = O * alpha + P V; final O / l -> fp16.
 #include <hip/hip_runtime.h>
+#include <type_traits>
+#include <utility>
 
 #ifndef DECA_BR
 #error "flash_attn.hip is a template: define the DECA_* macros"
@@ -90,6 +94,16 @@ typedef __attribute__((address_space(3))) void* lptr;
 // [BC][D]: chunk c of row r sits at c ^ ((r & 3) << 2), which rotates the 4 key
 // rows of one transposing read onto different 64-byte groups.
 
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>), in order
+template <class F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(f, std::make_integer_sequence<int, (N > 0 ? N : 0)>{});
+}
+
 #define DECA_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (((n) >> 4) << 14) | 0x0F70)
 
 extern "C" __global__ void __launch_bounds__(NT)
@@ -109,15 +123,28 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
   // fetched into one L2 only and shared there by all of its query tiles.
   constexpr int NQ = DECA_SQ / BR;
   constexpr int TOTAL = NQ * DECA_B * DECA_H;
+#if DECA_CAUSAL
+  // Query tiles near the end see the most keys.  They are scheduled first
+  // (flash_attn_tir.py:152-156), and first across all the (batch, head) slices
+  // that share an XCD rather than slice by slice: with the longest workgroups of
+  // every slice dispatched before any short one, the tail of the launch is made
+  // of short workgroups and the compute units finish together.
+  constexpr int BH = DECA_B * DECA_H;
+  int bh, qt;
+  if (BH % 8 == 0) {
+    constexpr int BHX = BH / 8 > 0 ? BH / 8 : 1;  // slices per XCD
+    const int idx = blockIdx.x >> 3;
+    bh = (blockIdx.x & 7) * BHX + idx % BHX;
+    qt = (NQ - 1) - idx / BHX;
+  } else {
+    bh = blockIdx.x % BH;
+    qt = (NQ - 1) - blockIdx.x / BH;
+  }
+  const int nkv = ((qt + 1) * BR + BC - 1) / BC;
+#else
   int lin = blockIdx.x;
   if (TOTAL % 8 == 0) lin = (lin & 7) * (TOTAL / 8) + (lin >> 3);
   const int bh = lin / NQ;
-#if DECA_CAUSAL
-  // Query tiles near the end see the most keys; schedule them first
-  // (flash_attn_tir.py:152-156).
-  const int qt = (NQ - 1) - (lin % NQ);
-  const int nkv = ((qt + 1) * BR + BC - 1) / BC;
-#else
   const int qt = lin % NQ;
   const int nkv = NKV;
 #endif
@@ -445,6 +472,211 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
     for (int mq = 0; mq < MQ; ++mq) l_i[mq] = l_i[mq] * alpha[mq] + sum[mq];
   };
 
+#if DECA_PIPE == 2
+  // ---- slot-interleaved loop ----------------------------------------------------------------
+  // One iteration = NS slots, one matrix instruction (per query tile) each: first
+  // the S^T of tile j+1, then O^T += V_j^T P_j^T.  Every slot also carries a fixed
+  // share of the vector work, so that the vector ALU runs in the shadow of the
+  // matrix pipe instead of in a phase of its own: the O^T rescale (S^T slots),
+  // the exponentials of tile j in three skewed stages (scale-and-shift in slot
+  // t-1, exp2 in slot t, row sum and fp16 packing in slot t+1; they run ahead of
+  // the O^T slots that consume them), and the running max of tile j+1 (O^T slots).
+  // Nothing moves across a slot boundary; operand fragments are read from LDS two
+  // slots ahead.
+  static_assert(STAGES == 2, "two K and two V slots");
+  static_assert(KT % 2 == 0, "S^T chains are issued in pairs");
+  constexpr int S_SLOTS = KT * DK, PV_SLOTS = KK * DT, NS = S_SLOTS + PV_SLOTS;
+  constexpr int NE = KT * 16;             // scores per lane and query tile
+  constexpr int NM = KT * 8;              // max3 operations of the running max
+  constexpr int NR = DT * 16;             // O^T registers to rescale
+  constexpr int PVM = PV_SLOTS - 1;       // O^T slots that carry the running max
+  struct Sched {
+    static constexpr int ne_s() { return NE * 5 / 8; }          // exponentials under the S^T slots
+    static constexpr int pve() { return PV_SLOTS - DT - 2; }    // O^T slots carrying the rest
+    // scores exponentiated by the end of slot t
+    static constexpr int e_end(int t) {
+      if (t < 0) return 0;
+      if (t < S_SLOTS) return ((t + 1) * ne_s()) / S_SLOTS;
+      const int v = ne_s() + ((t - S_SLOTS + 1) * (NE - ne_s()) + pve() - 1) / pve();
+      return v < NE ? v : NE;
+    }
+    // the 8 scores of k-step kk are packed one slot after their exp2 and must be
+    // there before the first O^T slot of that k-step
+    static constexpr bool ok() {
+      if (pve() < 1) return false;
+      for (int kk = 0; kk < KK; ++kk)
+        if (e_end(S_SLOTS + kk * DT - 2) < 8 * (kk + 1)) return false;
+      return e_end(NS - 3) == NE;
+    }
+  };
+  static_assert(Sched::ok(), "the exponentials do not meet the O^T slots in time");
+  auto finish_stats = [&](float (&mx)[MQ]) {
+#pragma unroll
+    for (int mq = 0; mq < MQ; ++mq) {
+      const float mxx = fmaxf(mx[mq], __shfl_xor(mx[mq], 32, 64));
+      const float m_new = fmaxf(m_i[mq], mxx);
+      alpha[mq] = __builtin_amdgcn_exp2f((m_i[mq] - m_new) * SL2);
+      m_i[mq] = m_new;
+      msl[mq] = m_new * SL2;
+    }
+  };
+  half2v pf2[KK][MQ][4];
+  auto fused = [&](auto with_m, auto v_slot, floatx16 (&sc)[KT][MQ], floatx16 (&sn)[KT][MQ]) {
+    constexpr bool WITH_M = decltype(with_m)::value;  // running max of tile j+1 in the O^T slots
+    constexpr int VSLOT = decltype(v_slot)::value;  // V_j; K_{j+1} is in the other K slot
+    const unsigned char* k_lds = lds + (VSLOT ^ 1) * TILE_BYTES;
+    const unsigned char* v_lds = lds + (STAGES + VSLOT) * TILE_BYTES;
+    const floatx16 zero = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f,
+                           0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    // slot t < S_SLOTS: pair p of key blocks, k-step ks, block kt; else k-step kk, d block dt
+    auto read_frag = [&](auto tc) -> half8 {
+      constexpr int t = decltype(tc)::value;
+      if constexpr (t < S_SLOTS) {
+        constexpr int pr = t / (2 * DK), r = t % (2 * DK), ks = r / 2, kt = 2 * pr + r % 2;
+        return *reinterpret_cast<const half8*>(
+            k_lds + ((k_lane_base ^ static_cast<unsigned>(ks * 32)) + kt * 32 * CPR * 16));
+      } else {
+        constexpr int u = t - S_SLOTS, kk = u / DT, dt = u % DT;
+        const unsigned base = v_lane_base ^ static_cast<unsigned>((dt * 4 * 16) & (CPR * 16 - 1));
+        const half4 h0 = __builtin_bit_cast(half4, __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (lds_s4_ptr)(v_lds + (base + (kk * 16) * CPR * 16))));
+        const half4 h1 = __builtin_bit_cast(half4, __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (lds_s4_ptr)(v_lds + (base + (kk * 16 + 8) * CPR * 16))));
+        return __builtin_shufflevector(h0, h1, 0, 1, 2, 3, 4, 5, 6, 7);
+      }
+    };
+    float sum[MQ][2], mx[MQ];
+#pragma unroll
+    for (int mq = 0; mq < MQ; ++mq) sum[mq][0] = sum[mq][1] = 0.0f;
+    // An empty asm that reads and writes a register: the value has to exist at this
+    // point, which keeps the optimiser from sinking the operation that produces it
+    // out of its slot, towards its first real use.
+    auto pin = [](auto& v) { asm volatile("" : "+v"(v)); };
+    // the vector work of slot t (t = -1: the scale-and-shift that slot 0 needs)
+    auto valu = [&](auto tc) {
+      constexpr int t = decltype(tc)::value;
+#pragma unroll
+      for (int mq = 0; mq < MQ; ++mq) {
+        // row sum and packing of what slot t-1 exponentiated
+        static_for<Sched::e_end(t - 1) - Sched::e_end(t - 2)>([&](auto ic) {
+          constexpr int e = Sched::e_end(t - 2) + decltype(ic)::value;
+          sum[mq][e & 1] += sc[e / 16][mq][e % 16];
+          pin(sum[mq][e & 1]);
+          if constexpr (e & 1) {
+            typedef float float2v __attribute__((ext_vector_type(2)));
+            const float2v pr = {sc[e / 16][mq][e % 16 - 1], sc[e / 16][mq][e % 16]};
+            unsigned packed = __builtin_bit_cast(unsigned, __builtin_convertvector(pr, half2v));
+            pin(packed);
+            pf2[e / 8][mq][(e % 8) / 2] = __builtin_bit_cast(half2v, packed);
+          }
+        });
+        static_for<Sched::e_end(t) - Sched::e_end(t - 1)>([&](auto ic) {
+          constexpr int e = Sched::e_end(t - 1) + decltype(ic)::value;
+          sc[e / 16][mq][e % 16] = __builtin_amdgcn_exp2f(sc[e / 16][mq][e % 16]);
+        });
+        static_for<Sched::e_end(t + 1) - Sched::e_end(t)>([&](auto ic) {
+          constexpr int e = Sched::e_end(t) + decltype(ic)::value;
+          sc[e / 16][mq][e % 16] = __builtin_fmaf(sc[e / 16][mq][e % 16], SL2, -msl[mq]);
+        });
+        if constexpr (t >= 0 && t < S_SLOTS) {
+          constexpr int lo = (t * NR) / S_SLOTS, hi = ((t + 1) * NR) / S_SLOTS;
+          static_for<hi - lo>([&](auto ic) {
+            constexpr int i = lo + decltype(ic)::value;
+            o_acc[i / 16][mq][i % 16] *= alpha[mq];
+          });
+        }
+        if constexpr (WITH_M && t >= S_SLOTS && t - S_SLOTS < PVM) {
+          constexpr int u = t - S_SLOTS;
+          if constexpr (u == 0) mx[mq] = sn[0][mq][0];
+          constexpr int lo = (u * NM) / PVM, hi = ((u + 1) * NM) / PVM;
+          static_for<hi - lo>([&](auto ic) {
+            constexpr int i = lo + decltype(ic)::value;
+            mx[mq] = fmaxf(fmaxf(mx[mq], sn[i / 8][mq][(i % 8) * 2]), sn[i / 8][mq][(i % 8) * 2 + 1]);
+            pin(mx[mq]);
+          });
+        }
+      }
+    };
+    half8 frag[3];
+    frag[0] = read_frag(std::integral_constant<int, 0>{});
+    frag[1] = read_frag(std::integral_constant<int, 1>{});
+    valu(std::integral_constant<int, -1>{});
+    __builtin_amdgcn_sched_barrier(0);
+    static_for<NS>([&](auto tc) {
+      constexpr int t = decltype(tc)::value;
+      if constexpr (t + 2 < NS) frag[(t + 2) % 3] = read_frag(std::integral_constant<int, t + 2>{});
+      if constexpr (t < S_SLOTS) {
+        constexpr int pr = t / (2 * DK), r = t % (2 * DK), ks = r / 2, kt = 2 * pr + r % 2;
+#pragma unroll
+        for (int mq = 0; mq < MQ; ++mq)
+          sn[kt][mq] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+              frag[t % 3], qf[mq][ks], ks == 0 ? zero : sn[kt][mq], 0, 0, 0);
+      } else {
+        constexpr int u = t - S_SLOTS, kk = u / DT, dt = u % DT;
+#pragma unroll
+        for (int mq = 0; mq < MQ; ++mq) {
+          const half8 pfr = __builtin_shufflevector(
+              __builtin_shufflevector(pf2[kk][mq][0], pf2[kk][mq][1], 0, 1, 2, 3),
+              __builtin_shufflevector(pf2[kk][mq][2], pf2[kk][mq][3], 0, 1, 2, 3), 0, 1, 2, 3, 4, 5, 6, 7);
+          o_acc[dt][mq] = __builtin_amdgcn_mfma_f32_32x32x16_f16(frag[t % 3], pfr, o_acc[dt][mq], 0, 0, 0);
+        }
+      }
+      valu(tc);
+      __builtin_amdgcn_sched_barrier(0);
+    });
+#pragma unroll
+    for (int mq = 0; mq < MQ; ++mq) l_i[mq] = l_i[mq] * alpha[mq] + (sum[mq][0] + sum[mq][1]);
+    if (WITH_M) finish_stats(mx);
+  };
+  half8 pf[KK][MQ];
+  // tile j: softmax and second product; tile j+1: first product and row statistics
+  auto step = [&](auto cur_slot, floatx16 (&sc)[KT][MQ], floatx16 (&sn)[KT][MQ], int j) {
+    constexpr int cur = decltype(cur_slot)::value;  // == j % 2
+    wait_and_barrier();  // K_{j+1}, V_j landed; everyone is done with K_j and V_{j-1}
+    if (j + 2 < nkv) issue_k(j + 2, cur);
+    issue_v(j + 1, cur ^ 1);
+    // (the rescale is unconditional here: a factor of 1 is exact, and a second copy of
+    // the slot sequence without it costs more registers than the skipped work is worth)
+#if DECA_CAUSAL
+    // One copy of the slot sequence only (a second one costs registers): the
+    // running max stays out of the slots, and follows the mask.
+    fused(std::integral_constant<bool, false>{}, cur_slot, sc, sn);
+    mask_s(sn, j + 1);
+    row_stats(sn);
+#else
+    fused(std::integral_constant<bool, true>{}, cur_slot, sc, sn);
+#endif
+  };
+  auto tail = [&](floatx16 (&sc)[KT][MQ], int j) {
+    wait_and_barrier();
+    rescale_o();
+    exp_and_pack(sc, pf);
+    compute_pv(pf, j & 1);
+  };
+  issue_k(0, 0);
+  issue_v(0, 0);
+  if (nkv > 1) issue_k(1, 1);
+  floatx16 s_a[KT][MQ], s_b[KT][MQ];
+  wait_and_barrier();
+  compute_s(s_a, 0);
+  mask_s(s_a, 0);
+  row_stats(s_a);
+  {
+    int j = 0;
+    const std::integral_constant<int, 0> even;
+    const std::integral_constant<int, 1> odd;
+    for (; j + 2 < nkv; j += 2) {
+      step(even, s_a, s_b, j);
+      step(odd, s_b, s_a, j + 1);
+    }
+    if (j + 1 < nkv) {
+      step(even, s_a, s_b, j);
+      tail(s_b, j + 1);
+    } else {
+      tail(s_a, j);
+    }
+  }
+#else
   issue_k(0, 0);
   issue_v(0, 0);
   if (nkv > 1) issue_k(1, 1);
@@ -475,6 +707,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
   rescale_o();
   exp_and_pack(s_cur, pf);
   compute_pv(pf, (nkv - 1) & 1);
+#endif
 #else
   issue_k(0, 0);
   issue_v(0, 0);

@@ -40,7 +40,10 @@ class FAConfig:
     stages: int = 2  # K/V LDS ring depth
     q_in_smem: bool = False  # kept for the record format; Q always lives in VGPRs here
     swizzle: bool = True  # kept for the record format; the LDS layout is always swizzled
-    pipe: bool = False  # compute S^T of tile j+1 before the softmax of tile j
+    # 0: S^T, softmax, O^T of one tile after the other.  1: S^T of tile j+1 is computed
+    # before the softmax of tile j (two S^T accumulators).  2: as 1, and every matrix
+    # instruction of an iteration carries a fixed share of its vector work.
+    pipe: int = 0
 
     @property
     def threads(self) -> int:
@@ -53,7 +56,7 @@ class FAConfig:
         return (
             f"Br={self.Br},Bc={self.Bc},warps={self.num_warps},stages={self.stages},"
             f"q_smem={int(self.q_in_smem)},swz={int(self.swizzle)}"
-            + (",pipe=1" if self.pipe else "")
+            + (f",pipe={int(self.pipe)}" if self.pipe else "")
         )
 
 
@@ -75,6 +78,30 @@ def est_regs_per_thread(cfg: FAConfig, D: int) -> int:
     return o_acc + s_acc + p_h + q_frag + kv_frag + 4 * mq + 40
 
 
+def slot_schedule_ok(Bc: int, D: int) -> bool:
+    """Whether the slot-interleaved loop (`pipe == 2`) can be scheduled: the S^T chains are
+    issued in pairs, and the exponentials, spread over the matrix instructions at a fixed
+    rate, must be packed before the O^T instruction that consumes them (the same check as
+    `Sched::ok()` in the kernel)."""
+    kt, dk, kk, dt = Bc // 32, D // 16, Bc // 16, D // 32
+    if Bc % 64 or kt % 2:
+        return False
+    s_slots, pv_slots = kt * dk, kk * dt
+    ns, ne = s_slots + pv_slots, kt * 16
+    ne_s, pve = ne * 5 // 8, pv_slots - dt - 2
+    if pve < 1:
+        return False
+
+    def e_end(t: int) -> int:
+        if t < 0:
+            return 0
+        if t < s_slots:
+            return (t + 1) * ne_s // s_slots
+        return min(ne, ne_s + ((t - s_slots + 1) * (ne - ne_s) + pve - 1) // pve)
+
+    return all(e_end(s_slots + k * dt - 2) >= 8 * (k + 1) for k in range(kk)) and e_end(ns - 3) == ne
+
+
 def check_config(cfg: FAConfig, S_q: int, S_kv: int, D: int) -> None:
     assert D % 64 == 0, "head dim must be a multiple of 64"
     assert cfg.Br % (32 * cfg.num_warps) == 0
@@ -85,7 +112,9 @@ def check_config(cfg: FAConfig, S_q: int, S_kv: int, D: int) -> None:
     assert 2 * (cfg.Bc * cpr) // cfg.threads <= 63
     assert cfg.threads <= 1024
     assert cfg.stages in (1, 2)
+    assert int(cfg.pipe) in (0, 1, 2)
     assert not cfg.pipe or cfg.stages == 2
+    assert int(cfg.pipe) != 2 or slot_schedule_ok(cfg.Bc, D)
     assert not cfg.q_in_smem and cfg.swizzle
     assert smem_bytes(cfg, D) <= MAX_LDS
     assert est_regs_per_thread(cfg, D) <= 512

@@ -110,12 +110,22 @@ FA_CASES = [
     (1, 3, 128, 640, 128, False, FAConfig(64, 64, 2, 2)),   # S_q != S_kv
     (1, 1, 384, 128, 64, False, FAConfig(128, 128, 4, 1)),
     (1, 1, 128, 128, 128, True, FAConfig(32, 32, 1, 2)),
+    (2, 4, 512, 512, 64, True, FAConfig(128, 64, 4, 2)),    # causal, whole slices per XCD
+    (3, 8, 256, 256, 64, True, FAConfig(64, 64, 2, 2)),
     # S^T computed one tile ahead of the softmax
     (1, 2, 512, 512, 128, False, FAConfig(256, 64, 8, 2, pipe=True)),
     (1, 2, 512, 512, 128, True, FAConfig(256, 64, 8, 2, pipe=True)),
     (2, 2, 512, 512, 64, True, FAConfig(128, 128, 4, 2, pipe=True)),
     (1, 2, 256, 384, 128, False, FAConfig(128, 128, 4, 2, pipe=True)),
     (1, 1, 128, 64, 64, False, FAConfig(64, 64, 2, 2, pipe=True)),   # a single KV tile
+    # slot-interleaved loop: even and odd numbers of KV tiles, one and two query tiles per wave
+    (1, 2, 512, 512, 128, False, FAConfig(256, 64, 8, 2, pipe=2)),
+    (1, 2, 512, 512, 128, True, FAConfig(256, 64, 8, 2, pipe=2)),
+    (2, 2, 512, 512, 64, True, FAConfig(256, 128, 8, 2, pipe=2)),
+    (1, 2, 256, 384, 128, False, FAConfig(128, 128, 4, 2, pipe=2)),  # 3 KV tiles
+    (1, 2, 128, 192, 64, False, FAConfig(128, 64, 2, 2, pipe=2)),    # two query tiles per wave
+    (1, 1, 128, 64, 64, False, FAConfig(64, 64, 2, 2, pipe=2)),      # a single KV tile
+    (1, 1, 128, 128, 64, True, FAConfig(64, 64, 2, 2, pipe=2)),      # two KV tiles, no loop
 ]
 
 FA_FULL = [
@@ -123,6 +133,8 @@ FA_FULL = [
     (4, 16, 4096, 4096, 128, True, FAConfig(128, 64, 4, 2)),
     (4, 16, 4096, 4096, 64, False, FAConfig(128, 64, 4, 2)),
     (4, 16, 4096, 4096, 64, True, FAConfig(128, 64, 4, 2)),
+    (4, 16, 4096, 4096, 128, True, FAConfig(256, 128, 8, 2)),
+    (4, 16, 4096, 4096, 64, False, FAConfig(256, 128, 8, 2, pipe=2)),
 ]
 
 

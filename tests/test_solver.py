@@ -120,7 +120,7 @@ def test_flash_attn_configs_are_valid(D, S):
         assert (S // cfg.Br) * B * H >= ARCH.sm_nums
     want = set()
     for br, bc, nw, st, pipe in itertools.product((32, 64, 128, 256), (32, 64, 128), (1, 2, 4, 8),
-                                                   (1, 2), (False, True)):
+                                                   (1, 2), (0, 1, 2)):
         cfg = fa.FAConfig(br, bc, nw, st, pipe=pipe)
         try:
             fa.check_config(cfg, S, S, D)
@@ -154,3 +154,19 @@ def test_z3_backend_is_reported_missing():
         pytest.skip("z3 is installed")
     with pytest.raises(RuntimeError, match="z3"):
         Solver.solve_rowwise(ARCH, "softmax", 16384, 4096, backend="z3")
+
+
+def test_slot_interleaved_loop_needs_paired_key_blocks():
+    """`pipe == 2` issues the S^T chains in pairs of 32-key blocks and must fit the
+    exponentials ahead of the O^T instructions that consume them."""
+    assert all(fa.slot_schedule_ok(bc, d) for bc in (64, 128) for d in (64, 128))
+    assert not any(fa.slot_schedule_ok(bc, d) for bc in (32, 96) for d in (64, 128))
+    fa.check_config(fa.FAConfig(128, 64, 4, 2, pipe=2), 512, 512, 128)
+    with pytest.raises(AssertionError):
+        fa.check_config(fa.FAConfig(128, 32, 4, 2, pipe=2), 512, 512, 128)
+    with pytest.raises(AssertionError):
+        fa.check_config(fa.FAConfig(128, 64, 4, 1, pipe=2), 512, 512, 128)
+    assert str(fa.FAConfig(128, 64, 4, 2, pipe=2)).endswith(",pipe=2")
+    assert str(fa.FAConfig(128, 64, 4, 2, pipe=True)).endswith(",pipe=1")
+    picked = Solver.solve_flash_attn(ARCH, 4, 16, 4096, 4096, 128)
+    assert any(c.pipe == 2 for c in picked) and all(c.Bc % 64 == 0 for c in picked if c.pipe == 2)
