@@ -387,9 +387,11 @@ def _fa_constraints(arch, B: int, H: int, S_q: int, S_kv: int, D: int, type_size
         # registers: O^T accumulator + S^T accumulator + P + Q fragments + K/V fragments
         mq = o.udiv(br, nw * 32)
         o_acc = mq * (D // 32 * 16)
-        p_h = mq * o.udiv(bc, c(4))
-        # the pipelined loops keep two S^T tiles
-        s_acc = mq * o.udiv(bc, c(2)) * o.ite(o.uge(pipe, c(1)), c(2), c(1))
+        # two S^T tiles in the pipelined loop; in the slot-interleaved one, tile j's scores
+        # turn into packed halves while tile j+1's chains come to life
+        s_one = mq * o.udiv(bc, c(2))
+        s_acc = o.ite(o.eq(pipe, c(1)), s_one * 2, o.ite(o.eq(pipe, c(2)), o.udiv(s_one * 7, c(4)), s_one))
+        p_h = o.ite(o.eq(pipe, c(2)), o.udiv(mq * o.udiv(bc, c(4)), c(2)), mq * o.udiv(bc, c(4)))
         q_frag = mq * (D // 16 * 4)
         regs = o_acc + s_acc + p_h + q_frag + 16 + mq * 4 + 40
         regs8 = o.udiv(regs + 7, c(8)) * 8

@@ -71,8 +71,11 @@ def est_regs_per_thread(cfg: FAConfig, D: int) -> int:
     o_acc = (D // 32) * mq * 16
     s_acc = (cfg.Bc // 32) * mq * 16
     p_h = s_acc // 2
-    if cfg.pipe:
+    if int(cfg.pipe) == 1:
         s_acc *= 2
+    elif int(cfg.pipe) == 2:
+        # tile j's scores turn into packed halves while tile j+1's chains come to life
+        s_acc, p_h = s_acc * 7 // 4, p_h // 2
     q_frag = mq * (D // 16) * 4
     kv_frag = 2 * 4 * 2  # a few K / V fragments in flight
     return o_acc + s_acc + p_h + q_frag + kv_frag + 4 * mq + 40
