@@ -91,8 +91,25 @@ typedef __attribute__((address_space(3))) void* lptr;
 // LDS layouts.  K tile [BC][D]: 16-byte chunk c of row r sits at chunk slot
 // c ^ ((r / rows_per_window) & mask), so that 16 consecutive rows at one logical
 // chunk land on 16 different bank groups of the 256-byte bank window.  V tile
-// [BC][D]: chunk c of row r sits at c ^ ((r & 3) << 2), which rotates the 4 key
-// rows of one transposing read onto different 64-byte groups.
+// [BC][D]: chunk c of row r sits at c ^ v_swz(r), which puts the 4 key rows that
+// one half of a transposing read touches (64 bytes each) onto the 4 different
+// 64-byte groups of the 256-byte bank window: with 256-byte rows (D = 128) all
+// rows alias and the group is rotated by r % 4; with 128-byte rows (D = 64)
+// rows r and r + 1 already sit in different halves of the window, and rows r
+// and r + 2 are told apart by bit 1 of r.
+constexpr int v_swz(int row) {
+  return CPR >= 16 ? (((row & 3) << 2) & (CPR - 1)) : (((row >> 1) & 1) << 2);
+}
+
+// Slices per dispatch group of the causal kernel: the smallest divisor g of the
+// slices of an XCD with g * nq >= 32 workgroups (64 when a slice has 16 or more
+// query tiles).
+constexpr int causal_group(int nq, int bhx) {
+  const int want = nq >= 16 ? 64 : 32;
+  for (int g = 1; g < bhx; ++g)
+    if (bhx % g == 0 && g * nq >= want) return g;
+  return bhx;
+}
 
 // f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>), in order
 template <class F, int... I>
@@ -125,17 +142,23 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
   constexpr int TOTAL = NQ * DECA_B * DECA_H;
 #if DECA_CAUSAL
   // Query tiles near the end see the most keys.  They are scheduled first
-  // (flash_attn_tir.py:152-156), and first across all the (batch, head) slices
-  // that share an XCD rather than slice by slice: with the longest workgroups of
-  // every slice dispatched before any short one, the tail of the launch is made
-  // of short workgroups and the compute units finish together.
+  // (flash_attn_tir.py:152-156), and first across a group of G (batch, head)
+  // slices rather than slice by slice: with the longest workgroups of several
+  // slices dispatched before any short one, the short ones fill the gaps and the
+  // compute units of an XCD finish together.  G is the smallest group that gives
+  // every compute unit of the XCD (32) a workgroup, twice that for long rows; larger
+  // groups only spread the K/V working set over more slices than the L2 holds
+  // (measured at S = 1024 ... 4096: a few percent lost at either end).
   constexpr int BH = DECA_B * DECA_H;
   int bh, qt;
   if (BH % 8 == 0) {
     constexpr int BHX = BH / 8 > 0 ? BH / 8 : 1;  // slices per XCD
+    constexpr int G = causal_group(NQ, BHX);
+    static_assert(BHX % G == 0, "groups of whole slices");
     const int idx = blockIdx.x >> 3;
-    bh = (blockIdx.x & 7) * BHX + idx % BHX;
-    qt = (NQ - 1) - idx / BHX;
+    const int in = idx % (G * NQ);
+    bh = (blockIdx.x & 7) * BHX + (idx / (G * NQ)) * G + in % G;
+    qt = (NQ - 1) - in / G;
   } else {
     bh = blockIdx.x % BH;
     qt = (NQ - 1) - blockIdx.x / BH;
@@ -163,7 +186,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
     constexpr int ROWS_PER_WINDOW = (16 / CPR) > 0 ? (16 / CPR) : 1;
     constexpr int MASK = (CPR < 16 ? CPR : 16) - 1;
     const int ck = cs ^ ((row / ROWS_PER_WINDOW) & MASK);
-    const int cv = cs ^ (((row & 3) << 2) & (CPR - 1));
+    const int cv = cs ^ v_swz(row);
     k_voff[it] = static_cast<unsigned>(row * D_ + ck * 8) * 2u;
     v_voff[it] = static_cast<unsigned>(row * D_ + cv * 8) * 2u;
   }
@@ -227,7 +250,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
   const int v_row0 = (tb >> 1) * 4 + (ti >> 2);
   const int v_d0 = 16 * (tb & 1) + 4 * (ti & 3);
   const unsigned v_lane_base = static_cast<unsigned>(
-      v_row0 * CPR * 16 + (((v_d0 >> 3) ^ (((v_row0 & 3) << 2) & (CPR - 1))) * 16) +
+      v_row0 * CPR * 16 + (((v_d0 >> 3) ^ v_swz(v_row0)) * 16) +
       ((v_d0 >> 2) & 1) * 8);
   static_assert(CPR >= 8, "D >= 64");
   // ---- the three phases of one KV step ----------------------------------------------------
