@@ -52,6 +52,9 @@
 #ifndef DECA_EPI_LDS
 #define DECA_EPI_LDS 1
 #endif
+#ifndef DECA_MIN_WAVES
+#define DECA_MIN_WAVES 1  // waves per SIMD the register allocation must leave room for
+#endif
 
 constexpr int NT = NW * 64;
 constexpr int WQ = BR / NW;       // query rows per wave
@@ -123,7 +126,7 @@ __device__ __forceinline__ void static_for(F&& f) {
 
 #define DECA_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (((n) >> 4) << 14) | 0x0F70)
 
-extern "C" __global__ void __launch_bounds__(NT)
+extern "C" __global__ void __launch_bounds__(NT, DECA_MIN_WAVES)
 deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
           const _Float16* __restrict__ V, _Float16* __restrict__ O) {
   __shared__ __attribute__((aligned(16))) unsigned char lds[LDS_BYTES];

@@ -31,6 +31,9 @@
 #ifndef DECA_BM
 #error "gemm.hip is a template: define the DECA_* macros"
 #endif
+#ifndef DECA_MIN_WAVES
+#define DECA_MIN_WAVES 1  // waves per SIMD the register allocation must leave room for
+#endif
 #ifndef DECA_BF16
 #define DECA_BF16 0
 #endif
@@ -109,7 +112,7 @@ __device__ __forceinline__ int b_chunk_slot(int k, int c) {
   return k * CPR_B + (c ^ (((k & 3) << 2) & MASK));
 }
 
-extern "C" __global__ void __launch_bounds__(NT)
+extern "C" __global__ void __launch_bounds__(NT, DECA_MIN_WAVES)
 deca_main(const elem_t* __restrict__ A, const elem_t* __restrict__ B,
           elem_t* __restrict__ C) {
   __shared__ __attribute__((aligned(16))) unsigned char lds[LDS_BYTES];

@@ -81,6 +81,17 @@ def est_regs_per_thread(cfg: FAConfig, D: int) -> int:
     return o_acc + s_acc + p_h + q_frag + kv_frag + 4 * mq + 40
 
 
+def target_waves_per_simd(cfg: FAConfig, D: int) -> int:
+    """Waves per SIMD the kernel is compiled for: what the estimated registers and the LDS
+    footprint let co-reside.  Without it the compiler spends the whole 512-register file on
+    a workgroup of 4 waves or fewer (the only bound it knows is the block size), and a second
+    workgroup that the LDS has room for cannot share the SIMDs."""
+    regs8 = (est_regs_per_thread(cfg, D) + 7) // 8 * 8
+    by_regs = 512 // regs8
+    by_lds = (MAX_LDS // smem_bytes(cfg, D)) * cfg.num_warps // 4
+    return max(1, min(by_regs, by_lds, 8))
+
+
 def slot_schedule_ok(Bc: int, D: int) -> bool:
     """Whether the slot-interleaved loop (`pipe == 2`) can be scheduled: the S^T chains are
     issued in pairs, and the exponentials, spread over the matrix instructions at a fixed
@@ -138,6 +149,7 @@ def make_flash_attn_fwd(
         "DECA_BR": cfg.Br, "DECA_BC": cfg.Bc, "DECA_NW": cfg.num_warps,
         "DECA_STAGES": cfg.stages, "DECA_CAUSAL": int(causal),
         "DECA_SCALE": repr(float(scale)), "DECA_PIPE": int(cfg.pipe),
+        "DECA_MIN_WAVES": target_waves_per_simd(cfg, D),
     }
     return make_spec(
         TEMPLATE, defines, grid=((S_q // cfg.Br) * B * H, 1, 1), block=(cfg.threads, 1, 1), nargs=4,

@@ -95,6 +95,17 @@ def est_regs_per_thread(cfg: GemmConfig) -> int:
     return acc + 2 * frags + staging + 40
 
 
+def target_waves_per_simd(cfg: GemmConfig) -> int:
+    """Waves per SIMD the kernel is compiled for: what the estimated registers and the LDS
+    footprint let co-reside.  The compiler only knows the block size, and gives a workgroup
+    of 4 waves or fewer the whole 512-register file even when the LDS has room for a second
+    workgroup on the same SIMDs."""
+    regs8 = (est_regs_per_thread(cfg) + 7) // 8 * 8
+    by_regs = 512 // regs8
+    by_lds = (MAX_LDS // smem_bytes(cfg)) * (cfg.threads // WAVE) // 4
+    return max(1, min(by_regs, by_lds, 8))
+
+
 def check_config(cfg: GemmConfig, M: int, N: int, K: int, max_smem: int = MAX_LDS) -> None:
     assert cfg.stages in ((2, 3, 4) if cfg.direct else (1, 2))
     assert K // cfg.BK >= cfg.stages
@@ -132,6 +143,7 @@ def make_gemm_tc(M: int, N: int, K: int, cfg: GemmConfig, dtype: str = "float16"
         "DECA_STAGES": cfg.stages, "DECA_RASTER": cfg.raster,
         "DECA_EPI_LDS": int(cfg.epi_smem), "DECA_XCD": int(cfg.xcd),
         "DECA_DIRECT": int(cfg.direct), "DECA_BF16": int(dtype == "bfloat16"),
+        "DECA_MIN_WAVES": target_waves_per_simd(cfg),
     }
     return make_spec(
         TEMPLATE, defines, grid=((M // cfg.BM) * (N // cfg.BN), 1, 1), block=(cfg.threads, 1, 1),
