@@ -238,9 +238,9 @@ def fa_score(cfg, arch, shape, causal: bool = False) -> float:
       reads the whole K and V tile for its WQ query rows: 1 / WQ bytes per
       FLOP) vs. L2 time (every workgroup streams K/V once: 1 / Br bytes per
       FLOP); the non-bottleneck terms only partially overlap
-    - softmax: per score element one exponential (quarter rate) plus ~4 full
-      rate operations on the vector ALU, which runs beside the matrix cores
-      only when another wave on the SIMD has MFMAs to issue
+    - softmax: per score element one exponential plus ~4 full rate operations
+      on the vector ALU, which runs beside the matrix cores only when another
+      wave on the SIMD has MFMAs to issue (or the loop interleaves them itself)
     - wave efficiency: the tail of the last wave of workgroups is wasted
     - barriers: one per KV step, hidden better by several smaller resident
       workgroups (`arch.fa_cta_sync_penalty`)
@@ -265,9 +265,11 @@ def fa_score(cfg, arch, shape, causal: bool = False) -> float:
     t_valu = (8.0 / (4.0 * D)) * cus / valu_rate
     # share of the VALU work hidden under matrix work: by other waves on the SIMD,
     # or by the wave itself when its loop is software pipelined
-    overlap = min(1.0, max(0.0, waves_per_simd - 1.0) + (0.5 if cfg.pipe else 0.0))
+    # (measured on MI355X: only the slot-interleaved loop adds to what a second wave
+    # already hides, and even full overlap leaves ~40 % of the vector time exposed)
+    overlap = min(1.0, max(0.0, waves_per_simd - 1.0) + (0.25 if int(cfg.pipe) == 2 else 0.0))
     terms = sorted([t_mma, t_lds, t_l2])
-    t_flop = terms[-1] + 0.3 * (terms[0] + terms[1]) + (1.0 - 0.8 * overlap) * t_valu
+    t_flop = terms[-1] + 0.3 * (terms[0] + terms[1]) + (1.0 - 0.6 * overlap) * t_valu
     t_flop = max(t_flop, t_valu)
 
     pipe = 1.0 if cfg.stages >= 2 else 0.96
@@ -281,7 +283,10 @@ def fa_score(cfg, arch, shape, causal: bool = False) -> float:
         computed = sum(-(-(i + 1) * cfg.Br // cfg.Bc) * cfg.Bc for i in range(nq)) * cfg.Br
         useful = S_q * (S_q + 1) / 2 / computed
 
-    return wave_eff * pipe * sync * step * useful / (t_flop / t_mma)
+    # every further 32-query tile of a wave lengthens the dependent chain between barriers
+    chain = 1.0 / (1.0 + 0.05 * (wq // 32 - 1))
+
+    return wave_eff * pipe * sync * step * useful * chain / (t_flop / t_mma)
 
 
 def rank_fa_configs(configs, arch, shape, causal: bool = False, top_n: int | None = None):
