@@ -15,6 +15,7 @@
 //                       the current one (two S^T accumulators per wave)
 //                       2: as 1, and every matrix instruction of an iteration carries
 //                       a fixed share of the iteration's vector work ("slots")
+//   DECA_MIN_WAVES      waves per SIMD the register allocation leaves room for
 //
 // The problem is computed transposed, which is what makes the two MFMA
 // products chain without a layout change on CDNA:
