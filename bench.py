@@ -50,7 +50,10 @@ def workloads():
         w[name] = {"kind": "rowwise", "op": op, "M": M, "N": N, "dtype": dtype,
                    "cfg": _cfg(op, (M, N), dtype)}
     for n in (2048, 4096, 8192, 12288, 16384):
-        w[f"gemm_fp16_{n}"] = {"kind": "gemm", "M": n, "N": n, "K": n, "cfg": _cfg("GEMM", (n, n, n))}
+        w[f"gemm_fp16_{n}"] = {"kind": "gemm", "M": n, "N": n, "K": n, "dtype": "float16",
+                               "cfg": _cfg("GEMM", (n, n, n))}
+    w["gemm_bf16_8192"] = {"kind": "gemm", "M": 8192, "N": 8192, "K": 8192, "dtype": "bfloat16",
+                           "cfg": _cfg("GEMM", (8192, 8192, 8192), "bfloat16")}
     for D in (128, 64):
         for causal in (False, True):
             name = f"fa_fp16_b4h16s4096d{D}" + ("_causal" if causal else "")
@@ -73,7 +76,7 @@ def _spec(wl):
     if wl["kind"] == "gemm":
         from deca_amd.kernels.gemm_hip import make_gemm_tc
 
-        return make_gemm_tc(wl["M"], wl["N"], wl["K"], wl["cfg"])
+        return make_gemm_tc(wl["M"], wl["N"], wl["K"], wl["cfg"], wl["dtype"])
     if wl["kind"] == "fa":
         from deca_amd.kernels.flash_attn_hip import make_flash_attn_fwd
 
@@ -182,15 +185,17 @@ def run_gemm(wl, steps, warmup, with_cpu):
 
     M, N, K = wl["M"], wl["N"], wl["K"]
     kern = build_gemm_tc(_spec(wl))
-    a, b = make_inputs(M, N, K, seed=0, dist="uniform")
-    c = torch.empty(M, N, dtype=torch.float16, device="cuda")
+    tdt = torch.bfloat16 if wl["dtype"] == "bfloat16" else torch.float16
+    short = "bf16" if wl["dtype"] == "bfloat16" else "f16"
+    a, b = make_inputs(M, N, K, seed=0, dist="uniform", dtype=tdt)
+    c = torch.empty(M, N, dtype=tdt, device="cuda")
     wall, t_k = _timed_steps(kern, [(a, b, c)], steps, warmup)
     flops = gemm_flops(M, N, K)
     res = {
         "workload": wl["name"],
-        "metric": f"fp16 GEMM {M}x{N}x{K} (fp32 accumulate) TFLOPS",
+        "metric": f"{'bf16' if short == 'bf16' else 'fp16'} GEMM {M}x{N}x{K} (fp32 accumulate) TFLOPS",
         "value": flops / wall / 1e12, "unit": "TFLOP/s", "ms_per_step": wall * 1e3,
-        "dtype": "f16 in/out, f32 accumulate", "config": str(wl["cfg"]),
+        "dtype": f"{short} in/out, f32 accumulate", "config": str(wl["cfg"]),
         "roofline": {"bound": "mfma", "achieved": flops / t_k / 1e12, "peak": MFMA_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": flops / t_k / 1e12 / MFMA_PEAK_TFLOPS,
                      "traffic": None, "kernel_us": t_k * 1e6, "algorithmic_flops": flops},

@@ -205,7 +205,7 @@ def test_tuned_table_roundtrip(tmp_path):
     # the table shipped with the package covers every bench workload
     import bench
 
-    assert len(bench.workloads()) == 12
+    assert len(bench.workloads()) == 13
 
 
 def test_rotating_sets_and_cycle():
