@@ -170,3 +170,23 @@ def test_slot_interleaved_loop_needs_paired_key_blocks():
     assert str(fa.FAConfig(128, 64, 4, 2, pipe=True)).endswith(",pipe=1")
     picked = Solver.solve_flash_attn(ARCH, 4, 16, 4096, 4096, 128)
     assert any(c.pipe == 2 for c in picked) and all(c.Bc % 64 == 0 for c in picked if c.pipe == 2)
+
+
+def test_kernels_are_compiled_for_the_occupancy_the_estimates_allow():
+    """A workgroup of 4 waves or fewer must not be given the whole register file when the
+    LDS has room for a second one (DECA_MIN_WAVES)."""
+    from deca_amd.kernels import gemm_hip as gm
+
+    # D = 64: two 4-wave workgroups fit the LDS and 256 registers each
+    small = fa.FAConfig(256, 64, 4, 2)
+    assert fa.est_regs_per_thread(small, 64) <= 256 and fa.target_waves_per_simd(small, 64) == 2
+    # D = 128, 4 waves with two query tiles each: more than 256 registers -> one wave per SIMD
+    assert fa.target_waves_per_simd(fa.FAConfig(256, 64, 4, 2), 128) == 1
+    # 8 waves are two per SIMD by themselves; a 128 KiB ring leaves no room for more
+    assert fa.target_waves_per_simd(fa.FAConfig(256, 128, 8, 2), 128) == 2
+    spec = fa.make_flash_attn_fwd(1, 8, 512, 512, 64, small, None, False)
+    assert dict(spec.defines)["DECA_MIN_WAVES"] == 2
+    big = gm.GemmConfig(256, 256, 64, 128, 64, 2, 8, True, True, True)
+    assert gm.target_waves_per_simd(big) == 2
+    assert gm.target_waves_per_simd(gm.GemmConfig(128, 256, 64, 64, 128, 2, 8, True, True, True)) == 1
+    assert dict(gm.make_gemm_tc(4096, 4096, 4096, big).defines)["DECA_MIN_WAVES"] == 2
