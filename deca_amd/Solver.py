@@ -258,7 +258,7 @@ GEMM_DOMAINS = {
     "epi": (0, 1),
     "direct": (0, 1),
 }
-GEMM_RASTERS = (1, 2, 4, 8, 16)
+GEMM_RASTERS = (0, 1, 2, 4, 8, 16)  # 0: 16 x 16 blocks of tiles, 8 x 4 per XCD
 
 
 def _gemm_constraints(arch, M: int, N: int, K: int, type_size: int):
@@ -334,7 +334,11 @@ def solve_gemm_tc(arch, M: int, N: int, K: int, type_size: int = 2, count: int =
         # other constraints, so both are expanded here (reference: Solver.py:550-558).
         xcd = ((M // bm) * (N // bn)) % arch.num_xcd == 0
         for ras in GEMM_RASTERS:
-            if (M // bm) % ras == 0:
+            if ras == 0:
+                ok = xcd and (M // bm) % 16 == 0 and (N // bn) % 16 == 0
+            else:
+                ok = (M // bm) % ras == 0
+            if ok:
                 results.append(GemmConfig(BM=bm, BN=bn, BK=bk, warp_m=wm, warp_n=wn, stages=st,
                                           raster=ras, epi_smem=bool(epi), xcd=xcd,
                                           direct=bool(direct)))

@@ -126,6 +126,9 @@ def gemm_wave_dram_bytes_per_flop(cfg, arch, M: int, N: int, K: int, slots: int)
     if (M * K + K * N) * 2 <= 0.5 * cache:
         return (M * K + K * N) * 2 / (2.0 * M * N * K)
     GM, GN = M // cfg.BM, N // cfg.BN
+    if cfg.raster == 0:  # the tiles in flight form 16 x 16 blocks
+        blocks = max(1, math.ceil(min(slots, GM * GN) / 256))
+        return blocks * 16 * (cfg.BM + cfg.BN) / (min(slots, GM * GN) * cfg.BM * cfg.BN)
     g = cfg.raster
     cols = min(GN, math.ceil(slots / g))
     rows = min(GM, g * math.ceil(slots / (g * GN)))

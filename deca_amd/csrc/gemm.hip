@@ -8,7 +8,8 @@
 //
 //   DECA_M/N/K    problem size          DECA_BM/BN/BK  workgroup tile
 //   DECA_WM/WN    wave tile             DECA_STAGES    LDS ring depth (1 or 2)
-//   DECA_RASTER   workgroup rows per rasterisation group
+//   DECA_RASTER   workgroup rows per rasterisation group; 0: 16 x 16 blocks of tiles,
+//                 an 8 x 4 sub-block per XCD
 //   DECA_EPI_LDS  1: stage C through LDS for 16-byte stores
 //   DECA_XCD      1: remap workgroup ids so that each of the 8 XCDs (private L2)
 //                 owns a contiguous slab of tiles
@@ -77,7 +78,8 @@ static_assert(A_CHUNKS % NT == 0 && B_CHUNKS % NT == 0, "loader coverage");
 static_assert(NT >= 64 && NT <= 1024, "workgroup size");
 static_assert(STAGES >= 1 && STAGES <= 4, "LDS ring depth");
 static_assert(DECA_DIRECT == 0 || STAGES >= 2, "the direct-to-LDS ring needs two slots");
-static_assert(GM % DECA_RASTER == 0, "raster group must divide the workgroup rows");
+static_assert(DECA_RASTER == 0 || GM % (DECA_RASTER ? DECA_RASTER : 1) == 0,
+              "raster group must divide the workgroup rows");
 static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
 static_assert(CPR_B >= 8, "BN >= 64");
 
@@ -125,6 +127,27 @@ deca_main(const elem_t* __restrict__ A, const elem_t* __restrict__ B,
 
   // ---- workgroup -> tile mapping --------------------------------------------
   int lin = blockIdx.x;
+#if DECA_RASTER == 0
+  // Workgroups are dealt round-robin to the 8 XCDs.  The 256 workgroups in flight
+  // (one per CU) form a 16 x 16 block of tiles, of which every XCD takes an 8 x 4
+  // sub-block: its L2 fetches 12 operand panels for 32 tiles, and the 8 L2s
+  // together ask the fabric for only 16 A and 16 B panels per 256 tiles.  Blocks
+  // are walked row by row, back and forth, so that consecutive blocks share
+  // their A panels, or at the turn their B panels.
+  static_assert(GM % 16 == 0 && GN % 16 == 0, "16 x 16 blocks of tiles");
+  static_assert(DECA_XCD, "the block order is an XCD order");
+  int bm, bn;
+  {
+    const int x = lin & 7, idx = lin >> 3;
+    const int sb = idx >> 5, within = idx & 31;
+    constexpr int SBN = GN / 16;
+    const int sbr = sb / SBN;
+    int sbc = sb % SBN;
+    if (sbr & 1) sbc = SBN - 1 - sbc;
+    bm = sbr * 16 + (x >> 2) * 8 + (within & 7);
+    bn = sbc * 16 + (x & 3) * 4 + (within >> 3);
+  }
+#else
 #if DECA_XCD
   {
     // Workgroups are dealt round-robin to the 8 XCDs; give each XCD a
@@ -138,6 +161,7 @@ deca_main(const elem_t* __restrict__ A, const elem_t* __restrict__ B,
   constexpr int GROUP = DECA_RASTER * GN;
   const int bm = (lin / GROUP) * DECA_RASTER + (lin % GROUP) % DECA_RASTER;
   const int bn = (lin % GROUP) / DECA_RASTER;
+#endif
 
   const elem_t* a_gbase = A + static_cast<size_t>(bm) * BM * K_;
   const elem_t* b_gbase = B + static_cast<size_t>(bn) * BN;

@@ -45,7 +45,9 @@ class GemmConfig:
     warp_m: int = 128  # wave tile rows
     warp_n: int = 128  # wave tile columns
     stages: int = 2  # LDS ring depth: 2..4 with direct loads, 1..2 with VGPR staging
-    raster: int = 8  # workgroup rows per rasterisation group (1: plain row-major order)
+    # workgroup rows per rasterisation group (1: plain row-major order); 0: the tiles in
+    # flight form 16 x 16 blocks, of which every XCD takes an 8 x 4 sub-block
+    raster: int = 8
     epi_smem: bool = False  # stage C through LDS for 16-byte stores
     xcd: bool = True  # deal contiguous tile ranges to the 8 XCDs
     direct: bool = True  # global -> LDS loads that bypass the VGPRs (else VGPR-staged)
@@ -119,7 +121,10 @@ def check_config(cfg: GemmConfig, M: int, N: int, K: int, max_smem: int = MAX_LD
     # Every lane issues the same number of 16-byte loads for each operand.
     assert (cfg.BM * cfg.BK // 8) % cfg.threads == 0
     assert (cfg.BK * cfg.BN // 8) % cfg.threads == 0
-    assert (M // cfg.BM) % cfg.raster == 0
+    if cfg.raster == 0:
+        assert cfg.xcd and (M // cfg.BM) % 16 == 0 and (N // cfg.BN) % 16 == 0
+    else:
+        assert (M // cfg.BM) % cfg.raster == 0
     if cfg.xcd:
         assert ((M // cfg.BM) * (N // cfg.BN)) % 8 == 0
     if cfg.epi_smem:

@@ -68,6 +68,9 @@ GEMM_CASES = [
     (256, 256, 128, GemmConfig(64, 64, 64, 32, 32, 2, 1, False, False, True)),
     (128, 192, 64, GemmConfig(64, 64, 32, 32, 64, 2, 2, False, False, True)),
     (1024, 1024, 512, GemmConfig(256, 256, 32, 128, 128, 3, 4, False, True, True)),
+    # raster 0: 16 x 16 blocks of tiles, an 8 x 4 sub-block per XCD (one block; 2 x 2 blocks)
+    (1024, 1024, 128, GemmConfig(64, 64, 64, 32, 32, 2, 0, False, True, True)),
+    (2048, 2048, 64, GemmConfig(64, 64, 32, 32, 64, 2, 0, True, True, True)),
     # VGPR-staged ring
     (512, 512, 512, GemmConfig(256, 256, 64, 128, 128, 2, 1, False, False, False)),
     (512, 1024, 256, GemmConfig(256, 256, 32, 128, 128, 2, 2, True, True, False)),
@@ -80,6 +83,7 @@ GEMM_CASES = [
 GEMM_FULL = [
     (4096, 4096, 4096, GemmConfig(256, 256, 64, 128, 128, 2, 8, False, True, True)),
     (8192, 8192, 8192, GemmConfig(256, 256, 32, 128, 128, 3, 8, False, True, True)),
+    (8192, 8192, 8192, GemmConfig(256, 256, 64, 128, 64, 2, 0, True, True, True)),
 ]
 
 

@@ -78,7 +78,10 @@ def test_gemm_configs_are_valid(n):
     for cfg in configs:
         gm.check_config(cfg, n, n, n)
         assert (n // cfg.BM) * (n // cfg.BN) >= ARCH.sm_nums
-        assert (n // cfg.BM) % cfg.raster == 0
+        if cfg.raster == 0:  # 16 x 16 blocks of tiles, dealt to the XCDs as 8 x 4 sub-blocks
+            assert cfg.xcd and (n // cfg.BM) % 16 == 0 and (n // cfg.BN) % 16 == 0
+        else:
+            assert (n // cfg.BM) % cfg.raster == 0
         assert cfg.xcd == (((n // cfg.BM) * (n // cfg.BN)) % 8 == 0)
         assert cfg.stages >= 2 if cfg.direct else cfg.stages <= 2
     if n >= 4096:
@@ -104,6 +107,16 @@ def test_gemm_configs_are_valid(n):
         tiles.add((bm, bn, bk, wm, wn, st, epi, direct))
     got = {(c.BM, c.BN, c.BK, c.warp_m, c.warp_n, c.stages, c.epi_smem, c.direct) for c in configs}
     assert got == tiles
+    # every rasterisation that divides the grid is offered for every tile set
+    for c in configs:
+        gm_, gn_ = n // c.BM, n // c.BN
+        want = {r for r in (1, 2, 4, 8, 16) if gm_ % r == 0}
+        if c.xcd and gm_ % 16 == 0 and gn_ % 16 == 0:
+            want.add(0)
+        have = {d.raster for d in configs if (d.BM, d.BN, d.BK, d.warp_m, d.warp_n, d.stages, d.epi_smem, d.direct)
+                == (c.BM, c.BN, c.BK, c.warp_m, c.warp_n, c.stages, c.epi_smem, c.direct)}
+        assert have == want
+        break
 
 
 def test_gemm_rejects_shapes_no_tile_divides():
