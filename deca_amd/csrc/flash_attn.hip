@@ -738,26 +738,37 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
 #else
   issue_k(0, 0);
   issue_v(0, 0);
-  int slot = 0;
-  for (int j = 0; j < nkv; ++j) {
+#if STAGES == 2
+  // One KV step.  `slot` is a literal at both call sites, so that every LDS
+  // address of the step is "lane base + immediate" and needs no address arithmetic.
+  auto kv_step = [&](int j, int slot) __attribute__((always_inline)) {
     // Tile j has landed for every lane, and every wave is done with the slot
     // that tile j+1 is about to overwrite.
     wait_and_barrier();
-#if STAGES == 2
     if (j + 1 < nkv) {
       issue_k(j + 1, slot ^ 1);
       issue_v(j + 1, slot ^ 1);
     }
-#endif
     floatx16 s_acc[KT][MQ];
     half8 pf[KK][MQ];
     compute_s(s_acc, slot);
     mask_s(s_acc, j);
     softmax(s_acc, pf);
     compute_pv(pf, slot);
-#if STAGES == 2
-    slot ^= 1;
+  };
+  for (int j = 0; j < nkv; j += 2) {
+    kv_step(j, 0);
+    if (j + 1 < nkv) kv_step(j + 1, 1);
+  }
 #else
+  for (int j = 0; j < nkv; ++j) {
+    wait_and_barrier();
+    floatx16 s_acc[KT][MQ];
+    half8 pf[KK][MQ];
+    compute_s(s_acc, 0);
+    mask_s(s_acc, j);
+    softmax(s_acc, pf);
+    compute_pv(pf, 0);
     // single slot: everyone must be done reading before the refill
     __builtin_amdgcn_s_waitcnt(0xC07F);
     __builtin_amdgcn_s_barrier();
@@ -765,8 +776,8 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
       issue_k(j + 1, 0);
       issue_v(j + 1, 0);
     }
-#endif
   }
+#endif
 #endif
 
   // ---- epilogue: O[q][d] = O^T[d][q] / l ----------------------------------------------
