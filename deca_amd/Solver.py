@@ -423,6 +423,8 @@ def solve_flash_attn(arch, B: int, H: int, S_q: int, S_kv: int, D: int, type_siz
     """
     from deca_amd.kernels.flash_attn_hip import FAConfig
 
+    if D not in (64, 128, 256):  # the kernel's LDS swizzles need a power-of-two head dim
+        return []
     cons = _fa_constraints(arch, B, H, S_q, S_kv, D, type_size, max_est_regs)
     return [FAConfig(Br=br, Bc=bc, num_warps=nw, stages=st, pipe=int(pipe))
             for br, bc, nw, st, pipe in _enumerate(FA_DOMAINS, cons, count, backend)]

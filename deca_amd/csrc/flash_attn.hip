@@ -74,7 +74,8 @@ constexpr float LOG2E = 1.4426950408889634f;
 constexpr float NEG_INF = -1e30f;
 constexpr float SL2 = static_cast<float>(DECA_SCALE) * LOG2E;
 
-static_assert(D_ % 64 == 0, "head dim must be a multiple of 64");
+static_assert(D_ == 64 || D_ == 128 || D_ == 256,
+              "head dim: the XOR swizzles of the LDS layouts need a power of two >= 64");
 static_assert(BR % (32 * NW) == 0, "each wave owns a multiple of 32 query rows");
 static_assert(BC % 32 == 0, "BC must be a multiple of 32");
 static_assert(DECA_SQ % BR == 0 && DECA_SKV % BC == 0, "tiles must divide the sequences");

@@ -117,7 +117,9 @@ def slot_schedule_ok(Bc: int, D: int) -> bool:
 
 
 def check_config(cfg: FAConfig, S_q: int, S_kv: int, D: int) -> None:
-    assert D % 64 == 0, "head dim must be a multiple of 64"
+    # reference: D % 64 == 0 (flash_attn_tir.py:71); the XOR swizzles of the LDS layouts here
+    # need a power of two as well
+    assert D in (64, 128, 256), "head dim must be 64, 128 or 256"
     assert cfg.Br % (32 * cfg.num_warps) == 0
     assert cfg.Bc % 32 == 0
     assert S_q % cfg.Br == 0 and S_kv % cfg.Bc == 0

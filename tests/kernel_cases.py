@@ -114,6 +114,8 @@ FA_CASES = [
     (1, 3, 128, 640, 128, False, FAConfig(64, 64, 2, 2)),   # S_q != S_kv
     (1, 1, 384, 128, 64, False, FAConfig(128, 128, 4, 1)),
     (1, 1, 128, 128, 128, True, FAConfig(32, 32, 1, 2)),
+    (1, 2, 256, 256, 256, False, FAConfig(128, 64, 4, 2)),  # D = 256
+    (1, 1, 256, 256, 256, True, FAConfig(64, 32, 2, 2)),
     (2, 4, 512, 512, 64, True, FAConfig(128, 64, 4, 2)),    # causal, whole slices per XCD
     (3, 8, 256, 256, 64, True, FAConfig(64, 64, 2, 2)),
     # S^T computed one tile ahead of the softmax

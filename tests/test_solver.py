@@ -203,3 +203,15 @@ def test_kernels_are_compiled_for_the_occupancy_the_estimates_allow():
     assert gm.target_waves_per_simd(big) == 2
     assert gm.target_waves_per_simd(gm.GemmConfig(128, 256, 64, 64, 128, 2, 8, True, True, True)) == 1
     assert dict(gm.make_gemm_tc(4096, 4096, 4096, big).defines)["DECA_MIN_WAVES"] == 2
+
+
+def test_flash_attn_head_dims():
+    """64, 128 and 256 are supported; other multiples of 64 (which the reference accepts,
+    flash_attn_tir.py:71) have no LDS layout here and yield no config instead of a bad one."""
+    assert Solver.solve_flash_attn(ARCH, 4, 16, 2048, 2048, 192) == []
+    wide = Solver.solve_flash_attn(ARCH, 4, 16, 2048, 2048, 256)
+    assert wide
+    for cfg in wide:
+        fa.check_config(cfg, 2048, 2048, 256)
+    with pytest.raises(AssertionError):
+        fa.check_config(fa.FAConfig(128, 64, 4, 2), 2048, 2048, 192)
