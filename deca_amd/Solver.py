@@ -305,6 +305,10 @@ def _gemm_constraints(arch, M: int, N: int, K: int, type_size: int):
         waves_per_simd = o.udiv(waves + (simds - 1), c(simds))
         out += [o.ule(regs, c(arch.vgprs_per_simd)),
                 o.ule(regs8 * waves_per_simd, c(arch.vgprs_per_simd))]
+        # the loads of the (st - 2) youngest tiles stay in flight across a wait: the
+        # vector-memory counter holds 6 bits
+        out.append(o.implies(o.all_of(o.eq(direct, c(1)), o.uge(st, c(3))),
+                             o.ule((st - 2) * chunks, c(63))))
         # enough workgroups to give every CU at least one
         out.append(o.uge(o.udiv(m_, bm) * o.udiv(n_, bn), c(arch.sm_nums)))
         return out

@@ -121,6 +121,10 @@ def check_config(cfg: GemmConfig, M: int, N: int, K: int, max_smem: int = MAX_LD
     # Every lane issues the same number of 16-byte loads for each operand.
     assert (cfg.BM * cfg.BK // 8) % cfg.threads == 0
     assert (cfg.BK * cfg.BN // 8) % cfg.threads == 0
+    if cfg.direct:
+        # loads left in flight by the (stages - 2) youngest tiles fit the 6-bit counter
+        loads = (cfg.BM * cfg.BK + cfg.BK * cfg.BN) // 8 // cfg.threads
+        assert (cfg.stages - 2) * loads <= 63
     if cfg.raster == 0:
         assert cfg.xcd and (M // cfg.BM) % 16 == 0 and (N // cfg.BN) % 16 == 0
     else:

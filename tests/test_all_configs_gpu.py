@@ -1,0 +1,115 @@
+"""Every configuration the solvers emit for a few small shapes, run once on the
+GPU against torch's fp32 result of the same operator.
+
+This compiles several hundred code objects (minutes of host time), so it only
+runs when DECA_ALL_CONFIGS=1 is set; the regular GPU suite covers a hand-picked
+subset (kernel_cases.py).  Gates are the ones of the other GPU tests.
+"""
+
+import os
+from concurrent.futures import ThreadPoolExecutor
+
+import pytest
+import torch
+
+pytestmark = [
+    pytest.mark.gpu,
+    pytest.mark.skipif(os.environ.get("DECA_ALL_CONFIGS") != "1",
+                       reason="opt-in: compiles every solver configuration (set DECA_ALL_CONFIGS=1)"),
+]
+
+FA_SHAPES = [(2, 16, 1024, 64, False), (2, 16, 1024, 64, True), (2, 16, 1024, 128, False),
+             (2, 16, 1024, 128, True), (1, 16, 2048, 256, True)]
+GEMM_SHAPES = [(2048, 2048, 2048)]
+ROW_SHAPES = [("softmax", 2048, 4096, "float16"), ("rmsnorm", 2048, 8192, "bfloat16"),
+              ("softmax", 512, 32000, "float16"), ("rmsnorm", 512, 128256, "float16")]
+GEMM_STRIDE = int(os.environ.get("DECA_ALL_CONFIGS_GEMM_STRIDE", "7"))  # 1: every GEMM config
+
+
+def _build_all(specs):
+    from deca_amd.kernels.build import cached_build
+
+    with ThreadPoolExecutor(max_workers=min(16, os.cpu_count() or 1)) as pool:
+        return list(pool.map(cached_build, specs))
+
+
+def _arch():
+    from deca_amd.arch.MI355X import MI355X
+
+    return MI355X()
+
+
+@pytest.mark.parametrize("B,H,S,D,causal", FA_SHAPES)
+def test_every_flash_attn_config(B, H, S, D, causal):
+    from deca_amd import Solver
+    from deca_amd.driver.driver import load_kernel
+    from deca_amd.kernels.attn_bench import make_qkv, math_attention
+    from deca_amd.kernels.flash_attn_hip import make_flash_attn_fwd
+
+    configs = Solver.solve_flash_attn(_arch(), B, H, S, S, D)
+    specs = [make_flash_attn_fwd(B, H, S, S, D, cfg, None, causal) for cfg in configs]
+    paths = _build_all(specs)
+    q, k, v = make_qkv(B, H, S, S, D)
+    ref = math_attention(q, k, v, causal)
+    wrong = []
+    for cfg, spec, path in zip(configs, specs, paths):
+        o = torch.full_like(q, float("nan"))
+        load_kernel(spec, path)(q, k, v, o)
+        torch.cuda.synchronize()
+        err = (o.float() - ref).abs().max().item()
+        if not err <= 2e-3:
+            wrong.append((str(cfg), err))
+    assert not wrong, wrong
+
+
+@pytest.mark.parametrize("M,N,K", GEMM_SHAPES)
+def test_every_gemm_config(M, N, K):
+    from deca_amd import Solver
+    from deca_amd.driver.driver import load_kernel
+    from deca_amd.kernels.gemm_bench import make_inputs
+    from deca_amd.kernels.gemm_hip import make_gemm_tc
+
+    configs = Solver.solve_gemm_tc(_arch(), M, N, K)[::GEMM_STRIDE]
+    specs = [make_gemm_tc(M, N, K, cfg) for cfg in configs]
+    paths = _build_all(specs)
+    a, b = make_inputs(M, N, K)
+    ref = a.float() @ b.float()
+    scale = ref.abs().max().item()
+    wrong = []
+    for cfg, spec, path in zip(configs, specs, paths):
+        c = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
+        load_kernel(spec, path)(a, b, c)
+        torch.cuda.synchronize()
+        err = (c.float() - ref).abs().max().item() / scale
+        if not err <= 1e-2:
+            wrong.append((str(cfg), err))
+    assert not wrong, wrong
+
+
+@pytest.mark.parametrize("op,M,N,dtype", ROW_SHAPES)
+def test_every_rowwise_config(op, M, N, dtype):
+    from deca_amd import Solver
+    from deca_amd.driver.driver import load_kernel
+    from deca_amd.kernels.rowwise_bench import make_inputs
+    from deca_amd.kernels.rowwise_hip import make_rowwise
+
+    configs = Solver.solve_rowwise(_arch(), op, M, N)
+    specs = [make_rowwise(op, M, N, dtype, cfg, 1e-6) for cfg in configs]
+    paths = _build_all(specs)
+    inputs = make_inputs(op, M, N, dtype, std=2.0 if op == "softmax" else 1.0)
+    x = inputs[0].float()
+    if op == "softmax":
+        ref = torch.softmax(x, -1)
+    else:
+        normed = (x * torch.rsqrt((x * x).mean(-1, keepdim=True) + 1e-6)).to(inputs[0].dtype).float()
+        ref = normed * inputs[1].float()
+    tol = 1e-2 if dtype == "bfloat16" else 2e-3
+    wrong = []
+    for cfg, spec, path in zip(configs, specs, paths):
+        y = torch.full_like(inputs[0], float("nan"))
+        load_kernel(spec, path)(*inputs, y)
+        torch.cuda.synchronize()
+        err = ((y.float() - ref).abs() / ref.abs().clamp(min=1.0)).max().item()
+        if not err <= tol:
+            wrong.append((str(cfg), err))
+    assert not wrong, wrong
