@@ -328,7 +328,9 @@ def solve_gemm_tc(arch, M: int, N: int, K: int, type_size: int = 2, count: int =
     Returns:
         list of GemmConfig
     """
-    from deca_amd.kernels.gemm_hip import GemmConfig
+    from dataclasses import replace
+
+    from deca_amd.kernels.gemm_hip import GemmConfig, check_config
 
     tiles = _enumerate(GEMM_DOMAINS, _gemm_constraints(arch, M, N, K, type_size), count, backend)
     results = []
@@ -343,9 +345,16 @@ def solve_gemm_tc(arch, M: int, N: int, K: int, type_size: int = 2, count: int =
             else:
                 ok = (M // bm) % ras == 0
             if ok:
-                results.append(GemmConfig(BM=bm, BN=bn, BK=bk, warp_m=wm, warp_n=wn, stages=st,
-                                          raster=ras, epi_smem=bool(epi), xcd=xcd,
-                                          direct=bool(direct)))
+                cfg = GemmConfig(BM=bm, BN=bn, BK=bk, warp_m=wm, warp_n=wn, stages=st,
+                                 raster=ras, epi_smem=bool(epi), xcd=xcd, direct=bool(direct))
+                results.append(cfg)
+                # a grid that leaves a partial last wave may split its tiles in four
+                split = replace(cfg, tail=True, xcd=True)
+                try:
+                    check_config(split, M, N, K)
+                except AssertionError:
+                    continue
+                results.append(split)
     return results[:count]
 
 

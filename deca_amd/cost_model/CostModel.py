@@ -171,6 +171,13 @@ def gemm_tc_score(cfg, arch, M: int, N: int, K: int) -> float:
     slots = arch.sm_nums * wgs
     grid = (M // cfg.BM) * (N // cfg.BN)
     wave_eff = _wave_efficiency(grid, slots)
+    if getattr(cfg, "tail", False):
+        # the partial last wave runs as quarter tiles: a quarter of the work each, at the
+        # lower efficiency of the small tile (measured ~0.3 of a full tile's time)
+        from deca_amd.kernels.gemm_hip import tail_tiles
+
+        r = tail_tiles(cfg, M, N)
+        wave_eff = (grid / slots) / ((grid - r) / slots + math.ceil(4 * r / slots) * 0.32)
     waves_per_simd = wgs * cfg.num_warps / arch.simds_per_cu
     hiding = min(1.0, 0.82 + 0.09 * min(waves_per_simd, 2.0)) if waves_per_simd >= 1 else \
         0.82 * waves_per_simd

@@ -12,6 +12,7 @@ from __future__ import annotations
 
 import hashlib
 import os
+import re
 import shutil
 import subprocess
 import tempfile
@@ -57,10 +58,17 @@ class KernelSpec:
         return [f"-D{k}={v}" for k, v in self.defines]
 
     def key(self) -> str:
-        """Content hash: template text + macros + options."""
+        """Content hash: template text (with the csrc files it includes) + macros + options."""
         h = hashlib.sha1()
         with open(self.source_path, "rb") as f:
-            h.update(f.read())
+            text = f.read()
+        h.update(text)
+        # files of csrc/ that the template includes are part of the kernel's source
+        for name in re.findall(rb'^#include "([^"]+)"', text, re.M):
+            inc = os.path.join(CSRC_DIR, name.decode())
+            if os.path.exists(inc):
+                with open(inc, "rb") as f:
+                    h.update(f.read())
         h.update(repr((self.defines, self.options, BASE_OPTIONS)).encode())
         return h.hexdigest()[:20]
 

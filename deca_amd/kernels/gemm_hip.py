@@ -51,6 +51,10 @@ class GemmConfig:
     epi_smem: bool = False  # stage C through LDS for 16-byte stores
     xcd: bool = True  # deal contiguous tile ranges to the 8 XCDs
     direct: bool = True  # global -> LDS loads that bypass the VGPRs (else VGPR-staged)
+    # the tiles of the partial last wave of workgroups are split into four quarter tiles
+    # (BM/2 x BN/2, wave tiles halved), so that they fill the whole GPU for a quarter of
+    # a tile's time instead of a quarter of the GPU for a whole one
+    tail: bool = False
 
     @property
     def num_warps(self) -> int:
@@ -69,6 +73,7 @@ class GemmConfig:
             f"stages={self.stages},raster={self.raster},epi_smem={int(self.epi_smem)}"
             + ("" if self.xcd else ",xcd=0")
             + ("" if self.direct else ",direct=0")
+            + (",tail=1" if self.tail else "")
         )
 
 
@@ -95,6 +100,28 @@ def est_regs_per_thread(cfg: GemmConfig) -> int:
     # direct loads keep one offset register per chunk, staged loads four data registers
     staging = chunks if cfg.direct else chunks * 4
     return acc + 2 * frags + staging + 40
+
+
+NUM_CUS = 256  # gfx950 (MI355X)
+
+
+def resident_workgroups(cfg: GemmConfig) -> int:
+    """Workgroups of this config one CU holds at a time (registers, LDS, 32 wave slots)."""
+    regs8 = (est_regs_per_thread(cfg) + 7) // 8 * 8
+    waves = cfg.threads // WAVE
+    by_regs = (512 // regs8) // -(-waves // 4)
+    return max(1, min(by_regs, MAX_LDS // smem_bytes(cfg), 32 // waves))
+
+
+def tail_tiles(cfg: GemmConfig, M: int, N: int) -> int:
+    """Tiles of the partial last wave: what is left when the grid is dealt to the
+    workgroup slots of the whole GPU."""
+    return ((M // cfg.BM) * (N // cfg.BN)) % (NUM_CUS * resident_workgroups(cfg))
+
+
+def tail_stages(cfg: GemmConfig) -> int:
+    """Ring depth of the quarter tiles: twice the slots fit the same LDS."""
+    return min(4 if cfg.direct else 2, 2 * cfg.stages)
 
 
 def target_waves_per_simd(cfg: GemmConfig) -> int:
@@ -125,12 +152,27 @@ def check_config(cfg: GemmConfig, M: int, N: int, K: int, max_smem: int = MAX_LD
         # loads left in flight by the (stages - 2) youngest tiles fit the 6-bit counter
         loads = (cfg.BM * cfg.BK + cfg.BK * cfg.BN) // 8 // cfg.threads
         assert (cfg.stages - 2) * loads <= 63
+    if cfg.tail:
+        r = tail_tiles(cfg, M, N)
+        tiles = (M // cfg.BM) * (N // cfg.BN)
+        assert cfg.raster != 0 and 0 < r < tiles
+        assert not cfg.xcd or (tiles - r) % 8 == 0
+        assert (cfg.warp_m // 2) % MFMA_M == 0 and (cfg.warp_n // 2) % MFMA_M == 0 and cfg.BN // 2 >= 64
+        assert (cfg.BM // 2 * cfg.BK // 8) % cfg.threads == 0
+        assert (cfg.BK * (cfg.BN // 2) // 8) % cfg.threads == 0
+        assert not cfg.epi_smem or (cfg.BM // 2 * (cfg.BN // 2) // 8) % cfg.threads == 0
+        qs = tail_stages(cfg)
+        assert K // cfg.BK >= qs
+        if cfg.direct:
+            q_loads = (cfg.BM // 2 * cfg.BK + cfg.BK * (cfg.BN // 2)) // 8 // cfg.threads
+            assert (qs - 2) * q_loads <= 63
     if cfg.raster == 0:
         assert cfg.xcd and (M // cfg.BM) % 16 == 0 and (N // cfg.BN) % 16 == 0
     else:
         assert (M // cfg.BM) % cfg.raster == 0
-    if cfg.xcd:
-        assert ((M // cfg.BM) * (N // cfg.BN)) % 8 == 0
+    if cfg.xcd:  # the remap permutes the full tiles
+        full = (M // cfg.BM) * (N // cfg.BN) - (tail_tiles(cfg, M, N) if cfg.tail else 0)
+        assert full % 8 == 0
     if cfg.epi_smem:
         assert (cfg.BM * cfg.BN // 8) % cfg.threads == 0
     assert est_regs_per_thread(cfg) <= MAX_VGPRS
@@ -154,8 +196,14 @@ def make_gemm_tc(M: int, N: int, K: int, cfg: GemmConfig, dtype: str = "float16"
         "DECA_DIRECT": int(cfg.direct), "DECA_BF16": int(dtype == "bfloat16"),
         "DECA_MIN_WAVES": target_waves_per_simd(cfg),
     }
+    workgroups = (M // cfg.BM) * (N // cfg.BN)
+    if cfg.tail:
+        r = tail_tiles(cfg, M, N)
+        defines["DECA_TAIL"] = r
+        defines["DECA_TAIL_STAGES"] = tail_stages(cfg)
+        workgroups += 3 * r
     return make_spec(
-        TEMPLATE, defines, grid=((M // cfg.BM) * (N // cfg.BN), 1, 1), block=(cfg.threads, 1, 1),
+        TEMPLATE, defines, grid=(workgroups, 1, 1), block=(cfg.threads, 1, 1),
         nargs=3, options=FAST_MATH_OPTIONS, meta={"cfg": str(cfg), "dtype": dtype},
     )
 

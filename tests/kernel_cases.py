@@ -71,7 +71,11 @@ GEMM_CASES = [
     # raster 0: 16 x 16 blocks of tiles, an 8 x 4 sub-block per XCD (one block; 2 x 2 blocks)
     (1024, 1024, 128, GemmConfig(64, 64, 64, 32, 32, 2, 0, False, True, True)),
     (2048, 2048, 64, GemmConfig(64, 64, 32, 32, 64, 2, 0, True, True, True)),
+    # tail: the 64 tiles of the partial last wave (576 = 512 + 64) as 256 quarter tiles
+    (3072, 3072, 256, GemmConfig(128, 128, 64, 64, 64, 2, 4, True, True, True, True)),
+    (3072, 3072, 256, GemmConfig(128, 128, 64, 64, 64, 2, 1, False, True, True, True)),
     # VGPR-staged ring
+    (3840, 3840, 128, GemmConfig(128, 128, 64, 64, 64, 1, 2, True, True, False, True)),  # tail
     (512, 512, 512, GemmConfig(256, 256, 64, 128, 128, 2, 1, False, False, False)),
     (512, 1024, 256, GemmConfig(256, 256, 32, 128, 128, 2, 2, True, True, False)),
     (512, 512, 512, GemmConfig(128, 128, 32, 64, 32, 1, 4, True, True, False)),
@@ -84,6 +88,7 @@ GEMM_FULL = [
     (4096, 4096, 4096, GemmConfig(256, 256, 64, 128, 128, 2, 8, False, True, True)),
     (8192, 8192, 8192, GemmConfig(256, 256, 32, 128, 128, 3, 8, False, True, True)),
     (8192, 8192, 8192, GemmConfig(256, 256, 64, 128, 64, 2, 0, True, True, True)),
+    (6144, 6144, 6144, GemmConfig(256, 256, 64, 128, 64, 2, 8, True, True, True, True)),
 ]
 
 

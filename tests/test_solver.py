@@ -215,3 +215,28 @@ def test_flash_attn_head_dims():
         fa.check_config(cfg, 2048, 2048, 256)
     with pytest.raises(AssertionError):
         fa.check_config(fa.FAConfig(128, 64, 4, 2), 2048, 2048, 192)
+
+
+def test_gemm_tail_split_is_offered_where_a_partial_wave_remains():
+    """6144^3 with 256 x 256 tiles: 576 tiles = 2 waves of 256 + 64; the 64 may run as 256
+    quarter tiles.  A grid that fills its waves exactly gets no such variant."""
+    cfgs = Solver.solve_gemm_tc(ARCH, 6144, 6144, 6144)
+    split = [c for c in cfgs if c.tail]
+    assert split and all(str(c).endswith(",tail=1") for c in split)
+    big = gm.GemmConfig(256, 256, 64, 128, 64, 2, 8, True, True, True, tail=True)
+    assert big in split and gm.tail_tiles(big, 6144, 6144) == 64
+    spec = gm.make_gemm_tc(6144, 6144, 6144, big)
+    assert spec.grid == (512 + 4 * 64, 1, 1)
+    assert dict(spec.defines)["DECA_TAIL"] == 64 and dict(spec.defines)["DECA_TAIL_STAGES"] == 4
+    for c in split:
+        gm.check_config(c, 6144, 6144, 6144)
+        assert c.raster != 0 and 0 < gm.tail_tiles(c, 6144, 6144)
+    # 8192^3 with the same tile: 1024 tiles = 4 full waves
+    with pytest.raises(AssertionError):
+        gm.check_config(big, 8192, 8192, 8192)
+    assert not any(c.tail and (c.BM, c.BN) == (256, 256) for c in Solver.solve_gemm_tc(ARCH, 8192, 8192, 8192))
+    # the cost model prefers the split at 6144 and scores a config without tail as before
+    from deca_amd.cost_model import CostModel as cm
+
+    plain = gm.GemmConfig(256, 256, 64, 128, 64, 2, 8, True, True, True)
+    assert cm.gemm_tc_score(big, ARCH, 6144, 6144, 6144) > cm.gemm_tc_score(plain, ARCH, 6144, 6144, 6144)
