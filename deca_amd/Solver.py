@@ -258,7 +258,7 @@ GEMM_DOMAINS = {
     "epi": (0, 1),
     "direct": (0, 1),
 }
-GEMM_RASTERS = (0, 1, 2, 4, 8, 16)  # 0: 16 x 16 blocks of tiles, 8 x 4 per XCD
+GEMM_RASTERS = (0, 1, 2, 4, 8, 16)  # 0: 8 x 4 sub-blocks of tiles per XCD, neighbours in flight
 
 
 def _gemm_constraints(arch, M: int, N: int, K: int, type_size: int):
@@ -340,21 +340,20 @@ def solve_gemm_tc(arch, M: int, N: int, K: int, type_size: int = 2, count: int =
         # other constraints, so both are expanded here (reference: Solver.py:550-558).
         xcd = ((M // bm) * (N // bn)) % arch.num_xcd == 0
         for ras in GEMM_RASTERS:
-            if ras == 0:
-                ok = xcd and (M // bm) % 16 == 0 and (N // bn) % 16 == 0
-            else:
-                ok = (M // bm) % ras == 0
-            if ok:
-                cfg = GemmConfig(BM=bm, BN=bn, BK=bk, warp_m=wm, warp_n=wn, stages=st,
-                                 raster=ras, epi_smem=bool(epi), xcd=xcd, direct=bool(direct))
-                results.append(cfg)
-                # a grid that leaves a partial last wave may split its tiles in four
-                split = replace(cfg, tail=True, xcd=True)
-                try:
-                    check_config(split, M, N, K)
-                except AssertionError:
-                    continue
-                results.append(split)
+            if ras != 0 and (M // bm) % ras != 0:
+                continue
+            cfg = GemmConfig(BM=bm, BN=bn, BK=bk, warp_m=wm, warp_n=wn, stages=st,
+                             raster=ras, epi_smem=bool(epi), xcd=xcd or ras == 0,
+                             direct=bool(direct))
+            # a grid that leaves a partial last wave may split its tiles in four; the
+            # block order (raster 0) needs whole rounds of 8 sub-blocks of 8 x 4 tiles
+            for cand in (cfg, replace(cfg, tail=True, xcd=True)):
+                if ras == 0 or cand.tail:
+                    try:
+                        check_config(cand, M, N, K)
+                    except AssertionError:
+                        continue
+                results.append(cand)
     return results[:count]
 
 

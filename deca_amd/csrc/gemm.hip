@@ -8,8 +8,8 @@
 //
 //   DECA_M/N/K    problem size          DECA_BM/BN/BK  workgroup tile
 //   DECA_WM/WN    wave tile             DECA_STAGES    LDS ring depth (1 or 2)
-//   DECA_RASTER   workgroup rows per rasterisation group; 0: 16 x 16 blocks of tiles,
-//                 an 8 x 4 sub-block per XCD
+//   DECA_RASTER   workgroup rows per rasterisation group; 0: an 8 x 4 sub-block of
+//                 tiles per XCD, 8 neighbouring sub-blocks in flight
 //   DECA_EPI_LDS  1: stage C through LDS for 16-byte stores
 //   DECA_XCD      1: remap workgroup ids so that each of the 8 XCDs (private L2)
 //                 owns a contiguous slab of tiles
@@ -113,7 +113,6 @@ constexpr int LDS_BYTES = full_tile::LDS_BYTES;
 #endif
 static_assert(DECA_RASTER == 0 || GM % (DECA_RASTER ? DECA_RASTER : 1) == 0,
               "raster group must divide the workgroup rows");
-static_assert(DECA_TAIL == 0 || DECA_RASTER != 0, "the block order has no partial wave");
 static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
 
 extern "C" __global__ void __launch_bounds__(full_tile::NT, DECA_MIN_WAVES)
@@ -122,33 +121,53 @@ deca_main(const elem_t* __restrict__ A, const elem_t* __restrict__ B,
   __shared__ __attribute__((aligned(16))) unsigned char lds[LDS_BYTES];
 
   // ---- workgroup -> tile mapping --------------------------------------------
+  // With DECA_TAIL, workgroups TILES .. TILES + 4 * DECA_TAIL - 1 each take a quarter
+  // of one of the last DECA_TAIL tiles of the order below; they start as the full
+  // tiles of the last whole wave finish and fill the compute units that a partial
+  // wave of full tiles would leave idle.
   int lin = blockIdx.x;
-#if DECA_RASTER == 0
-  // Workgroups are dealt round-robin to the 8 XCDs.  The 256 workgroups in flight
-  // (one per CU) form a 16 x 16 block of tiles, of which every XCD takes an 8 x 4
-  // sub-block: its L2 fetches 12 operand panels for 32 tiles, and the 8 L2s
-  // together ask the fabric for only 16 A and 16 B panels per 256 tiles.  Blocks
-  // are walked row by row, back and forth, so that consecutive blocks share
-  // their A panels, or at the turn their B panels.
-  static_assert(GM % 16 == 0 && GN % 16 == 0, "16 x 16 blocks of tiles");
-  static_assert(DECA_XCD, "the block order is an XCD order");
+  int quarter = -1;
   int bm, bn;
+#if DECA_RASTER == 0
+  // Workgroups are dealt round-robin to the 8 XCDs.  Each XCD works on an 8 x 4
+  // sub-block of tiles at a time (32 workgroups, one per CU: its L2 fetches 12
+  // operand panels for 32 tiles), and the 8 sub-blocks in flight are neighbours:
+  // sub-blocks are numbered down two rows of sub-blocks at a time, so that 8
+  // consecutive ones form a 16 x 16 block of tiles and the 8 L2s together ask the
+  // fabric for only 16 A and 16 B panels per 256 tiles.  The two-row bands are
+  // walked back and forth, so that consecutive blocks share their A panels, or at
+  // the turn their B panels; an odd last row of sub-blocks is walked on its own.
+  static_assert(GM % 8 == 0 && GN % 4 == 0, "8 x 4 sub-blocks of tiles");
+  static_assert(TILES % 256 == 0, "whole rounds of 8 sub-blocks (the rest is the tail)");
+  static_assert(DECA_XCD, "the block order is an XCD order");
   {
-    const int x = lin & 7, idx = lin >> 3;
-    const int sb = idx >> 5, within = idx & 31;
-    constexpr int SBN = GN / 16;
-    const int sbr = sb / SBN;
-    int sbc = sb % SBN;
-    if (sbr & 1) sbc = SBN - 1 - sbc;
-    bm = sbr * 16 + (x >> 2) * 8 + (within & 7);
-    bn = sbc * 16 + (x & 3) * 4 + (within >> 3);
+    int sq, within;
+    if (DECA_TAIL && lin >= TILES) {
+      const int t = lin - TILES;
+      quarter = t & 3;
+      sq = TILES / 32 + (t >> 7);
+      within = (t >> 2) & 31;
+    } else {
+      const int x = lin & 7, idx = lin >> 3;
+      sq = (idx >> 5) * 8 + x;
+      within = idx & 31;
+    }
+    constexpr int NB = GM / 8, NC = GN / 4;  // sub-block rows and columns
+    constexpr int PAIR = 2 * NC;              // sub-blocks of a two-row band
+    const int band = sq / PAIR;
+    int sr, sc;
+    if (band < NB / 2) {
+      sr = 2 * band + (sq % PAIR & 1);
+      sc = (sq % PAIR) >> 1;
+    } else {
+      sr = NB - 1;
+      sc = sq - (NB / 2) * PAIR;
+    }
+    if (band & 1) sc = NC - 1 - sc;
+    bm = sr * 8 + (within & 7);
+    bn = sc * 4 + (within >> 3);
   }
 #else
-  // With DECA_TAIL, workgroups TILES .. TILES + 4 * DECA_TAIL - 1 each take a quarter
-  // of one of the last DECA_TAIL tiles (in rasterisation order); they start as the
-  // full tiles of the last whole wave finish and fill the compute units that a
-  // partial wave of full tiles would leave idle.
-  int quarter = -1;
   if (DECA_TAIL && lin >= TILES) {
     quarter = (lin - TILES) & 3;
     lin = TILES + ((lin - TILES) >> 2);
@@ -161,9 +180,11 @@ deca_main(const elem_t* __restrict__ A, const elem_t* __restrict__ B,
     lin = (lin & 7) * (TILES / 8) + (lin >> 3);
 #endif
   }
-  constexpr int GROUP = DECA_RASTER * GN;
-  const int bm = (lin / GROUP) * DECA_RASTER + (lin % GROUP) % DECA_RASTER;
-  const int bn = (lin % GROUP) / DECA_RASTER;
+  {
+    constexpr int GROUP = DECA_RASTER * GN;
+    bm = (lin / GROUP) * DECA_RASTER + (lin % GROUP) % DECA_RASTER;
+    bn = (lin % GROUP) / DECA_RASTER;
+  }
 #endif
 
 #if DECA_TAIL

@@ -45,8 +45,8 @@ class GemmConfig:
     warp_m: int = 128  # wave tile rows
     warp_n: int = 128  # wave tile columns
     stages: int = 2  # LDS ring depth: 2..4 with direct loads, 1..2 with VGPR staging
-    # workgroup rows per rasterisation group (1: plain row-major order); 0: the tiles in
-    # flight form 16 x 16 blocks, of which every XCD takes an 8 x 4 sub-block
+    # workgroup rows per rasterisation group (1: plain row-major order); 0: every XCD works
+    # on an 8 x 4 sub-block of tiles, and the 8 sub-blocks in flight are neighbours
     raster: int = 8
     epi_smem: bool = False  # stage C through LDS for 16-byte stores
     xcd: bool = True  # deal contiguous tile ranges to the 8 XCDs
@@ -155,7 +155,7 @@ def check_config(cfg: GemmConfig, M: int, N: int, K: int, max_smem: int = MAX_LD
     if cfg.tail:
         r = tail_tiles(cfg, M, N)
         tiles = (M // cfg.BM) * (N // cfg.BN)
-        assert cfg.raster != 0 and 0 < r < tiles
+        assert 0 < r < tiles
         assert not cfg.xcd or (tiles - r) % 8 == 0
         assert (cfg.warp_m // 2) % MFMA_M == 0 and (cfg.warp_n // 2) % MFMA_M == 0 and cfg.BN // 2 >= 64
         assert (cfg.BM // 2 * cfg.BK // 8) % cfg.threads == 0
@@ -167,7 +167,8 @@ def check_config(cfg: GemmConfig, M: int, N: int, K: int, max_smem: int = MAX_LD
             q_loads = (cfg.BM // 2 * cfg.BK + cfg.BK * (cfg.BN // 2)) // 8 // cfg.threads
             assert (qs - 2) * q_loads <= 63
     if cfg.raster == 0:
-        assert cfg.xcd and (M // cfg.BM) % 16 == 0 and (N // cfg.BN) % 16 == 0
+        full = (M // cfg.BM) * (N // cfg.BN) - (tail_tiles(cfg, M, N) if cfg.tail else 0)
+        assert cfg.xcd and (M // cfg.BM) % 8 == 0 and (N // cfg.BN) % 4 == 0 and full % 256 == 0
     else:
         assert (M // cfg.BM) % cfg.raster == 0
     if cfg.xcd:  # the remap permutes the full tiles

@@ -68,7 +68,10 @@ GEMM_CASES = [
     (256, 256, 128, GemmConfig(64, 64, 64, 32, 32, 2, 1, False, False, True)),
     (128, 192, 64, GemmConfig(64, 64, 32, 32, 64, 2, 2, False, False, True)),
     (1024, 1024, 512, GemmConfig(256, 256, 32, 128, 128, 3, 4, False, True, True)),
-    # raster 0: 16 x 16 blocks of tiles, an 8 x 4 sub-block per XCD (one block; 2 x 2 blocks)
+    # raster 0: an 8 x 4 sub-block of tiles per XCD, 8 neighbours in flight (one round; four
+    # rounds; an odd number of sub-block rows; with the tail split)
+    (3072, 4096, 128, GemmConfig(128, 128, 64, 64, 64, 2, 0, False, True, True)),
+    (3072, 3072, 256, GemmConfig(128, 128, 64, 64, 64, 2, 0, True, True, True, True)),
     (1024, 1024, 128, GemmConfig(64, 64, 64, 32, 32, 2, 0, False, True, True)),
     (2048, 2048, 64, GemmConfig(64, 64, 32, 32, 64, 2, 0, True, True, True)),
     # tail: the 64 tiles of the partial last wave (576 = 512 + 64) as 256 quarter tiles

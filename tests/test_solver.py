@@ -78,11 +78,12 @@ def test_gemm_configs_are_valid(n):
     for cfg in configs:
         gm.check_config(cfg, n, n, n)
         assert (n // cfg.BM) * (n // cfg.BN) >= ARCH.sm_nums
-        if cfg.raster == 0:  # 16 x 16 blocks of tiles, dealt to the XCDs as 8 x 4 sub-blocks
-            assert cfg.xcd and (n // cfg.BM) % 16 == 0 and (n // cfg.BN) % 16 == 0
+        full = (n // cfg.BM) * (n // cfg.BN) - (gm.tail_tiles(cfg, n, n) if cfg.tail else 0)
+        if cfg.raster == 0:  # 8 x 4 sub-blocks of tiles per XCD, whole rounds of 8 of them
+            assert cfg.xcd and (n // cfg.BM) % 8 == 0 and (n // cfg.BN) % 4 == 0 and full % 256 == 0
         else:
             assert (n // cfg.BM) % cfg.raster == 0
-        assert cfg.xcd == (((n // cfg.BM) * (n // cfg.BN)) % 8 == 0)
+        assert cfg.xcd == (full % 8 == 0)
         assert cfg.stages >= 2 if cfg.direct else cfg.stages <= 2
     if n >= 4096:
         assert gm.GemmConfig(256, 256, 64, 128, 64, 2, 4, False, True, True) in configs
@@ -109,11 +110,14 @@ def test_gemm_configs_are_valid(n):
     assert got == tiles
     # every rasterisation that divides the grid is offered for every tile set
     for c in configs:
+        if c.tail:
+            continue
         gm_, gn_ = n // c.BM, n // c.BN
         want = {r for r in (1, 2, 4, 8, 16) if gm_ % r == 0}
-        if c.xcd and gm_ % 16 == 0 and gn_ % 16 == 0:
+        if gm_ % 8 == 0 and gn_ % 4 == 0 and (gm_ * gn_) % 256 == 0:
             want.add(0)
-        have = {d.raster for d in configs if (d.BM, d.BN, d.BK, d.warp_m, d.warp_n, d.stages, d.epi_smem, d.direct)
+        have = {d.raster for d in configs if not d.tail and
+                (d.BM, d.BN, d.BK, d.warp_m, d.warp_n, d.stages, d.epi_smem, d.direct)
                 == (c.BM, c.BN, c.BK, c.warp_m, c.warp_n, c.stages, c.epi_smem, c.direct)}
         assert have == want
         break
@@ -230,7 +234,8 @@ def test_gemm_tail_split_is_offered_where_a_partial_wave_remains():
     assert dict(spec.defines)["DECA_TAIL"] == 64 and dict(spec.defines)["DECA_TAIL_STAGES"] == 4
     for c in split:
         gm.check_config(c, 6144, 6144, 6144)
-        assert c.raster != 0 and 0 < gm.tail_tiles(c, 6144, 6144)
+        assert 0 < gm.tail_tiles(c, 6144, 6144)
+    assert gm.GemmConfig(256, 256, 64, 128, 64, 2, 0, True, True, True, tail=True) in split
     # 8192^3 with the same tile: 1024 tiles = 4 full waves
     with pytest.raises(AssertionError):
         gm.check_config(big, 8192, 8192, 8192)
