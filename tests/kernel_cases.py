@@ -100,6 +100,7 @@ GEMM_BF16_CASES = [
     (512, 512, 512, GemmConfig(256, 256, 64, 128, 64, 2, 1, False, False, True)),
     (512, 1024, 256, GemmConfig(128, 128, 32, 64, 64, 3, 2, True, True, True)),
     (256, 256, 192, GemmConfig(64, 64, 64, 32, 32, 1, 1, False, False, False)),
+    (3072, 3072, 256, GemmConfig(128, 128, 64, 64, 64, 2, 0, True, True, True, True)),  # block order + tail
 ]
 
 

@@ -20,7 +20,7 @@ pytestmark = [
 
 FA_SHAPES = [(2, 16, 1024, 64, False), (2, 16, 1024, 64, True), (2, 16, 1024, 128, False),
              (2, 16, 1024, 128, True), (1, 16, 2048, 256, True)]
-GEMM_SHAPES = [(2048, 2048, 2048)]
+GEMM_SHAPES = [(2048, 2048, 2048), (3072, 3072, 512)]  # the second leaves partial waves (tail)
 ROW_SHAPES = [("softmax", 2048, 4096, "float16"), ("rmsnorm", 2048, 8192, "bfloat16"),
               ("softmax", 512, 32000, "float16"), ("rmsnorm", 512, 128256, "float16")]
 GEMM_STRIDE = int(os.environ.get("DECA_ALL_CONFIGS_GEMM_STRIDE", "7"))  # 1: every GEMM config
