@@ -677,6 +677,10 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
   };
   auto tail = [&](floatx16 (&sc)[KT][MQ], int j) {
     wait_and_barrier();
+#if DECA_CAUSAL
+    // every key of the last tile lies after every query row of this wave: P = 0 exactly
+    if (j * BC > qt * BR + wave_u * WQ + WQ - 1) return;
+#endif
     rescale_o();
     exp_and_pack(sc, pf);
     compute_pv(pf, j & 1);
@@ -732,9 +736,15 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
   }
   // last tile: nothing left to prefetch
   wait_and_barrier();
-  rescale_o();
-  exp_and_pack(s_cur, pf);
-  compute_pv(pf, (nkv - 1) & 1);
+#if DECA_CAUSAL
+  // (unless every key of it lies after every query row of this wave: P = 0 exactly)
+  if ((nkv - 1) * BC <= qt * BR + wave_u * WQ + WQ - 1)
+#endif
+  {
+    rescale_o();
+    exp_and_pack(s_cur, pf);
+    compute_pv(pf, (nkv - 1) & 1);
+  }
 #endif
 #else
   issue_k(0, 0);
@@ -750,6 +760,14 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
       issue_k(j + 1, slot ^ 1);
       issue_v(j + 1, slot ^ 1);
     }
+#if DECA_CAUSAL
+    // Every key of the tile lies after every query row of this wave (the last tile
+    // of a workgroup with BR > BC): all its scores are masked, P = 0 exactly, and
+    // there is nothing to add.  (Skipping single masked 32-key blocks of the
+    // diagonal tiles as well was tried: the extra code paths cost registers and
+    // made the kernel slower.)
+    if (j * BC > qt * BR + wave_u * WQ + WQ - 1) return;
+#endif
     floatx16 s_acc[KT][MQ];
     half8 pf[KK][MQ];
     compute_s(s_acc, slot);
