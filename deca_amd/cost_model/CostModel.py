@@ -231,6 +231,9 @@ def rank_gemm_configs(configs, arch, M: int, N: int, K: int, top_n: int | None =
 # ---------------------------------------------------------------------------
 # FlashAttention forward
 # ---------------------------------------------------------------------------
+_FA_HIDDEN = 0.0  # share of a workgroup's start-up latency still exposed beside a second workgroup
+
+
 def fa_occupancy(cfg, arch, D: int, grid: int):
     """Returns (resident workgroups per CU, share of the wave slots in use)."""
     from deca_amd.kernels.flash_attn_hip import est_regs_per_thread, smem_bytes
@@ -296,7 +299,17 @@ def fa_score(cfg, arch, shape, causal: bool = False) -> float:
     # every further 32-query tile of a wave lengthens the dependent chain between barriers
     chain = 1.0 / (1.0 + 0.05 * (wq // 32 - 1))
 
-    return wave_eff * pipe * sync * step * useful * chain / (t_flop / t_mma)
+    # A workgroup starts with nothing in flight (Q, then the first K/V tile) and ends with
+    # the O store: a few microseconds that only another resident workgroup can cover.
+    # It matters when the KV loop is short (measured at S = 512: two 4-wave workgroups per
+    # CU beat one 8-wave workgroup by 20 %).  The constants are a compromise between that
+    # shape and S = 4096, D = 64, where a stronger term would rank 4-wave configs too high.
+    kv_len = S_kv * (0.5 if causal else 1.0)
+    t_loop = 4.0 * cfg.Br * kv_len * D / (0.42 * arch.peak_mma_sync_flops * 1e9 / cus)
+    exposed = getattr(arch, "fa_workgroup_latency_s", 2e-6) * (1.0 if wgs == 1 else _FA_HIDDEN)
+    ramp = t_loop / (t_loop + exposed)
+
+    return wave_eff * pipe * sync * step * useful * chain * ramp / (t_flop / t_mma)
 
 
 def rank_fa_configs(configs, arch, shape, causal: bool = False, top_n: int | None = None):

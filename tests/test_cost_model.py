@@ -94,7 +94,15 @@ def test_fa_score_terms():
     for i in range(nq):
         computed += math.ceil((i + 1) * 256 / 128) * 128 * 256
     ratio = cm.fa_score(one, ARCH, shape, True) / cm.fa_score(one, ARCH, shape, False)
-    assert ratio == pytest.approx(4096 * 4097 / 2 / computed)
+    # ... times the start-up latency of a workgroup, which weighs more on the halved KV loop
+    rate = 0.42 * ARCH.peak_mma_sync_flops * 1e9 / ARCH.sm_nums
+    t_full, lat = 4.0 * 256 * 4096 * 128 / rate, 2e-6
+    ramp = (t_full / 2 / (t_full / 2 + lat)) / (t_full / (t_full + lat))
+    assert ratio == pytest.approx(4096 * 4097 / 2 / computed * ramp)
+    # a short KV loop favours two resident workgroups over one that owns the CU
+    short = (32, 16, 512, 512, 128)
+    assert (cm.fa_score(FAConfig(128, 64, 4, 2), ARCH, short) / cm.fa_score(a, ARCH, short)
+            > cm.fa_score(FAConfig(128, 64, 4, 2), ARCH, shape) / cm.fa_score(a, ARCH, shape))
     wgs, share = cm.fa_occupancy(a, ARCH, 128, 1024)
     assert wgs == 1 and share == pytest.approx(8 / 32)
     assert cm.rank_fa_configs([FAConfig(32, 32, 1, 1), a], ARCH, shape, top_n=1) == [a]
