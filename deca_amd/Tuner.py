@@ -133,7 +133,9 @@ class Tuner:
 
         top = self.top_n or None
         if self.operator == "GEMM":
-            return cm.rank_gemm_configs(configs, self.arch, *shape, top_n=top)
+            # at most 3 tile orders per tile set among the measured candidates
+            return cm.rank_gemm_configs(configs, self.arch, *shape, top_n=top,
+                                        per_tile=3 if top else None)
         if self.operator in ("softmax", "rmsnorm"):
             return cm.rank_rowwise_configs(configs, self.arch, self.operator, *shape, top_n=top)
         return cm.rank_fa_configs(configs, self.arch, shape, causal, top_n=top)
