@@ -155,6 +155,7 @@ def gemm_tc_score(cfg, arch, M: int, N: int, K: int) -> float:
       (BM + BN) / (BM * BN) B/FLOP, from the L2 of its XCD; without the XCD remap
       neighbouring tiles land on different XCDs and share nothing there
     - HBM / Infinity Cache: the unique A / B blocks of one wave of workgroups
+    - fabric: the A / B blocks that the tiles in flight on one XCD miss in its L2
     Then:
     - wave efficiency of the workgroup grid
     - issue: with one wave per SIMD nothing covers that wave's own waits (LDS
@@ -193,7 +194,20 @@ def gemm_tc_score(cfg, arch, M: int, N: int, K: int) -> float:
     t_l2 = l2_bpf * cus / (arch.l2_bw * 1e9)
     dram_bpf = gemm_wave_dram_bytes_per_flop(cfg, arch, M, N, K, slots)
     t_dram = dram_bpf * cus / (arch.dram_bw * 1e9)
-    terms = sorted([t_mma, t_lds, t_l2, t_dram])
+    # L2 misses: what the tiles in flight on ONE XCD need from the fabric.  A banded order
+    # gives an XCD `raster` rows of tiles, the block order 8 rows by 4 columns per resident
+    # workgroup; an order that is not XCD-aware leaves neighbours on different L2s.
+    per_xcd = max(1, slots // getattr(arch, "num_xcd", 8))
+    if not cfg.xcd:
+        rows_x, cols_x = per_xcd, per_xcd
+    elif cfg.raster == 0:
+        rows_x, cols_x = 8, max(1, per_xcd // 8)
+    else:
+        rows_x = min(cfg.raster, per_xcd)
+        cols_x = min(N // cfg.BN, math.ceil(per_xcd / rows_x))
+    fabric_bpf = (rows_x * cfg.BM + cols_x * cfg.BN) / (per_xcd * cfg.BM * cfg.BN)
+    t_fabric = fabric_bpf * cus / (getattr(arch, "mall_bw", arch.l2_bw) * 1e9)
+    terms = sorted([t_mma, t_lds, t_l2, t_dram, t_fabric])
     t_flop = terms[-1] + 0.25 * sum(terms[:-1])
 
     # Bytes per CU that must be in flight to cover the L2 / fabric latency at the
