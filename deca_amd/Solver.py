@@ -192,11 +192,17 @@ def _rowwise_constraints(arch, op: str, M: int, N: int, type_size: int, force_re
             regs = o.udiv(elems * 9, c(8)) + 12
         else:
             regs = o.udiv(elems * 5, c(4)) + 16 + o.udiv(vec, c(2))
-        regs8 = o.udiv(regs + 7, c(8)) * 8
         waves_per_simd = o.udiv(o.udiv(threads, c(wave)) + (simds - 1), c(simds))
+
+        def fits(r):
+            return o.all_of(o.ule(r, c(arch.max_arch_vgprs)),
+                            o.ule(o.udiv(r + 7, c(8)) * 8 * waves_per_simd, c(arch.vgprs_per_simd)))
+
+        # reg mode falls back to its lean form (only the packed row stays in registers
+        # between the passes), as in rowwise_hip.use_lean
+        lean = o.udiv(chunks * vec * 5, c(8)) + 16
         out += [
-            o.ule(regs, c(arch.max_arch_vgprs)),
-            o.ule(regs8 * waves_per_simd, c(arch.vgprs_per_simd)),
+            o.any_of(fits(regs), o.all_of(o.eq(mode, c(0)), fits(lean))),
             # reg mode is fully unrolled; twopass needs one full loop iteration
             o.implies(o.eq(mode, c(0)), o.all_of(o.eq(unroll, c(1)), o.ule(chunks, c(32)))),
             o.implies(o.eq(mode, c(1)), o.ule(unroll, o.udiv(n, span))),

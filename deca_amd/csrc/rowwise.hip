@@ -14,6 +14,8 @@
 //   DECA_MODE    0 reg (row cached in VGPRs), 1 twopass (row streamed twice)
 //   DECA_UNROLL  chunks in flight per twopass iteration
 //   DECA_HINT    1: non-temporal loads of read-once data and non-temporal stores
+//   DECA_LEAN    1 (reg mode): nothing but the packed row stays in registers between
+//                the reduction and the stores -- the fp32 values are computed again
 //   DECA_EPS     RMSNorm epsilon
 //
 // Lane t of a row owns the VEC-element chunks (c * TPR + t) * VEC, so one wave
@@ -52,6 +54,10 @@ typedef __bf16 elem_t;
 typedef _Float16 elem_t;
 #endif
 typedef elem_t vec_t __attribute__((ext_vector_type(VEC)));
+
+#ifndef DECA_LEAN
+#define DECA_LEAN 0
+#endif
 
 #define LOG2E 1.4426950408889634f
 #define NEG_INF (-1e30f)
@@ -175,6 +181,11 @@ deca_main(const elem_t* __restrict__ x,
     for (int i = 0; i < VEC; ++i) m = fmaxf(m, ok ? static_cast<float>(xh[c][i]) : NEG_INF);
   }
   const float m2 = row_reduce(m, MaxOp(), red0, rb, wr, lane) * LOG2E;
+#if DECA_LEAN
+  // (see below: the fp32 conversions of the max pass are not kept for the sum)
+#pragma unroll
+  for (int c = 0; c < NCHUNK; ++c) asm volatile("" : "+v"(xh[c]));
+#endif
   float s = 0.0f;
 #pragma unroll
   for (int c = 0; c < NCHUNK; ++c) {
@@ -186,6 +197,13 @@ deca_main(const elem_t* __restrict__ x,
     }
   }
   const float inv = __builtin_amdgcn_rcpf(row_reduce(s, AddOp(), red1, rb, wr, lane));
+#if DECA_LEAN
+  // The optimiser would keep the exponentials of the sum alive for the stores
+  // (2 VGPRs per element on top of the packed row).  Reading the row through an
+  // opaque copy makes it compute them again from the same bits instead.
+#pragma unroll
+  for (int c = 0; c < NCHUNK; ++c) asm volatile("" : "+v"(xh[c]));
+#endif
 #pragma unroll
   for (int c = 0; c < NCHUNK; ++c) {
     if (in_row(c)) {
@@ -209,6 +227,11 @@ deca_main(const elem_t* __restrict__ x,
   }
   ss = row_reduce(ss, AddOp(), red0, rb, wr, lane);
   const float r = __builtin_amdgcn_rsqf(ss * (1.0f / DECA_N) + static_cast<float>(DECA_EPS));
+#if DECA_LEAN
+  // as above: the fp32 conversions of the row are made again, not kept
+#pragma unroll
+  for (int c = 0; c < NCHUNK; ++c) asm volatile("" : "+v"(xh[c]));
+#endif
 #pragma unroll
   for (int c = 0; c < NCHUNK; ++c) {
     if (in_row(c)) {

@@ -37,6 +37,7 @@ MODES = ("reg", "twopass")
 WAVE = 64
 MAX_VGPRS = 512  # unified VGPRs per lane available to a single wave
 VGPRS_PER_SIMD = 512
+MAX_ARCH_VGPRS = 256  # architectural VGPRs one wave can address
 MAX_THREADS = 1024
 TPR_CHOICES = (16, 32, 64, 128, 256, 512, 1024)
 TEMPLATE = "rowwise.hip"
@@ -85,6 +86,33 @@ def est_regs_per_thread(cfg: RowConfig, N: int, op: str) -> int:
     return elems * 5 // 4 + 16 + cfg.vec // 2
 
 
+def _fits(regs: int, threads: int) -> bool:
+    """One workgroup of `threads` lanes with `regs` VGPRs each fits the CU's 4 SIMDs."""
+    waves_per_simd = -(-(threads // WAVE) // 4)
+    # (these kernels have no use for the accumulation half of the unified register file)
+    return regs <= MAX_ARCH_VGPRS and (regs + 7) // 8 * 8 * waves_per_simd <= VGPRS_PER_SIMD
+
+
+def lean_regs_per_thread(cfg: RowConfig, N: int) -> int:
+    """Estimate for the lean form of the reg mode: only the packed row (E / 2) stays in
+    registers between the passes, the fp32 values are computed again (78 VGPRs measured at
+    E = 128 for softmax, 77-85 for RMSNorm)."""
+    elems = num_chunks(cfg, N) * cfg.vec
+    return elems * 5 // 8 + 16
+
+
+def use_lean(cfg: RowConfig, N: int, op: str) -> bool:
+    """The lean reg mode is compiled when the plain one would not fit its workgroup into
+    the register files: that is what lets a 128256-element row be read from HBM once."""
+    return (cfg.mode == "reg" and not _fits(est_regs_per_thread(cfg, N, op), cfg.threads)
+            and _fits(lean_regs_per_thread(cfg, N), cfg.threads))
+
+
+def regs_per_thread(cfg: RowConfig, N: int, op: str) -> int:
+    """Estimate of the form that gets compiled (plain or lean)."""
+    return lean_regs_per_thread(cfg, N) if use_lean(cfg, N, op) else est_regs_per_thread(cfg, N, op)
+
+
 def check_config(cfg: RowConfig, op: str, M: int, N: int, dtype: str) -> None:
     assert op in OPS and dtype in DTYPES and cfg.mode in MODES
     assert cfg.vec in (2, 4, 8) and N % cfg.vec == 0
@@ -96,11 +124,10 @@ def check_config(cfg: RowConfig, op: str, M: int, N: int, dtype: str) -> None:
     if cfg.mode == "twopass":
         # at least one full loop iteration
         assert cfg.unroll <= N // (cfg.threads_per_row * cfg.vec)
-    regs = est_regs_per_thread(cfg, N, op)
-    assert regs <= MAX_VGPRS
+    if cfg.mode == "reg":
+        assert num_chunks(cfg, N) <= 32  # the row loop is fully unrolled
     # one workgroup must fit in the register files of the CU's 4 SIMDs
-    waves_per_simd = -(-(cfg.threads // WAVE) // 4)
-    assert (regs + 7) // 8 * 8 * waves_per_simd <= VGPRS_PER_SIMD
+    assert _fits(regs_per_thread(cfg, N, op), cfg.threads)
 
 
 def make_rowwise(
@@ -125,6 +152,8 @@ def make_rowwise(
         "DECA_HINT": int(cfg.hint),
         "DECA_EPS": repr(float(eps)),
     }
+    if use_lean(cfg, N, op):
+        defines["DECA_LEAN"] = 1
     return make_spec(
         TEMPLATE, defines, grid=(M // cfg.rows_per_block, 1, 1), block=(cfg.threads, 1, 1),
         nargs=3 if op == "rmsnorm" else 2, options=FAST_MATH_OPTIONS,

@@ -25,6 +25,13 @@ ROWWISE_CASES = [
     ("softmax", 64, 32000, "float16", RowConfig(1024, 1, 8, "twopass", 2, True)),
     ("softmax", 64, 32000, "float16", RowConfig(1024, 1, 8, "reg")),
     ("softmax", 16, 128256, "bfloat16", RowConfig(1024, 1, 8, "twopass", 4)),
+    # lean reg mode: a vocabulary-size row cached in registers (only the packed row
+    # survives between the passes), and a short row over very few lanes
+    ("softmax", 32, 128256, "float16", RowConfig(1024, 1, 8, "reg", 1, True)),
+    ("softmax", 32, 128256, "bfloat16", RowConfig(512, 1, 8, "reg")),
+    ("rmsnorm", 32, 128256, "bfloat16", RowConfig(1024, 1, 8, "reg", 1, True)),
+    ("rmsnorm", 32, 128256, "float16", RowConfig(512, 1, 8, "reg")),
+    ("softmax", 512, 4096, "float16", RowConfig(16, 8, 8)),
     ("softmax", 256, 4096, "float16", RowConfig(64, 4, 8, "twopass", 2)),
     ("softmax", 256, 4096, "float16", RowConfig(128, 1, 4, "twopass", 1, True)),
     # single-row and single-block extremes

@@ -62,3 +62,28 @@ def test_compile_only_and_register_estimate(tmp_path):
     path = rw.build_rowwise_to_file("softmax", (64, 1024), "float16", RowConfig(64, 1, 8), 1e-6,
                                     "gfx950", str(tmp_path / "k.hsaco"))
     assert os.path.getsize(path) > 1000
+
+
+def test_lean_reg_mode_is_chosen_when_the_plain_one_does_not_fit(tmp_path):
+    """A 128256-element row over 1024 lanes is 128 elements per lane: the plain reg mode
+    (fp32 values kept between the passes) does not fit 16 waves into the register files,
+    the lean one (packed row only) does, and compiles without spills."""
+    cfg = RowConfig(1024, 1, 8, "reg", 1, True)
+    for op, dtype in (("softmax", "float16"), ("rmsnorm", "bfloat16")):
+        assert rw.use_lean(cfg, 128256, op) and not rw.use_lean(cfg, 32000, op)
+        rw.check_config(cfg, op, 4096, 128256, dtype)
+        spec = rw.make_rowwise(op, 4096, 128256, dtype, cfg)
+        assert dict(spec.defines)["DECA_LEAN"] == 1
+        res = kernel_resources(spec)
+        assert res["vgpr_spills"] == 0 and res["scratch_bytes"] == 0
+        assert res["vgprs"] <= rw.lean_regs_per_thread(cfg, 128256) <= 128
+    assert "DECA_LEAN" not in dict(rw.make_rowwise("softmax", 4096, 32000, "float16", cfg).defines)
+    # 64 chunks per lane are beyond the unrolled row loop
+    with pytest.raises(AssertionError):
+        rw.check_config(RowConfig(256, 1, 8, "reg"), "softmax", 4096, 128256, "float16")
+    # the solver offers the register-cached form for vocabulary-size rows
+    from deca_amd import Solver
+    from deca_amd.arch.MI355X import MI355X
+
+    cfgs = Solver.solve_rowwise(MI355X(), "softmax", 4096, 128256)
+    assert cfg in cfgs and any(c.mode == "twopass" for c in cfgs)

@@ -48,7 +48,7 @@ def test_rowwise_configs_are_valid_and_exhaustive(op, M, N):
             continue
         if mode == "reg" and (unroll != 1 or rw.num_chunks(cfg, N) > 32):
             continue
-        if rw.est_regs_per_thread(cfg, N, op) > ARCH.max_arch_vgprs:
+        if rw.regs_per_thread(cfg, N, op) > ARCH.max_arch_vgprs:
             continue
         want.add(cfg)
     has_reg = any(c.mode == "reg" for c in want)
