@@ -16,6 +16,8 @@
 //                       2: as 1, and every matrix instruction of an iteration carries
 //                       a fixed share of the iteration's vector work ("slots")
 //   DECA_MIN_WAVES      waves per SIMD the register allocation leaves room for
+//   DECA_LAZY_TAU       the running max follows a tile's max only when that is more
+//                       than this many powers of two above it (0: always)
 //
 // The problem is computed transposed, which is what makes the two MFMA
 // products chain without a layout change on CDNA:
@@ -36,7 +38,9 @@
 // value -1e30 on tiles crossing the diagonal only; m' = max(m, rowmax S);
 // alpha = exp2((m - m') * sl2); p = exp2(S * sl2 - m' * sl2), sl2 = scale * log2e;
 // l = l * alpha + sum p (fp32 p); P = fp16(p) feeds the second product;
-// O = O * alpha + P V; final O / l -> fp16.
+// O = O * alpha + P V; final O / l -> fp16.  One departure: m' is taken lazily
+// (DECA_LAZY_TAU), which leaves O / l the same quotient with p <= 2^tau
+// instead of p <= 1 and makes alpha exactly 1 for almost every tile.
 #include <hip/hip_runtime.h>
 #include <type_traits>
 #include <utility>
@@ -50,6 +54,9 @@
 #define BC DECA_BC
 #define NW DECA_NW
 #define STAGES DECA_STAGES
+#ifndef DECA_LAZY_TAU
+#define DECA_LAZY_TAU 8
+#endif
 #ifndef DECA_EPI_LDS
 #define DECA_EPI_LDS 1
 #endif
@@ -304,6 +311,19 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
     (void)j;
 #endif
   };
+  // The running max only follows the tile's max when that is more than
+  // DECA_LAZY_TAU powers of two above it (always for the first tile): until
+  // then p = exp2((S - m) * sl2) stays below 2^DECA_LAZY_TAU, which fp16 P and
+  // the fp32 sums hold as well as values below 1, and alpha is exactly 1, so
+  // the O^T rescale is skipped.  O / l at the end is the same quotient.
+  auto lazy_max = [&](float m_old, float mx) {
+    const float m_new = fmaxf(m_old, mx);
+#if DECA_LAZY_TAU > 0
+    return (m_new - m_old) * SL2 > static_cast<float>(DECA_LAZY_TAU) ? m_new : m_old;
+#else
+    return m_new;
+#endif
+  };
   // Online softmax of one tile: one query column per lane.  Leaves P^T (fp16,
   // already in operand order) in `pf` and rescales O^T when a running max moved
   // (skipped otherwise: multiplying by 1 is exact).
@@ -317,7 +337,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
 #pragma unroll
         for (int e = 0; e < 16; ++e) mx = fmaxf(mx, s_acc[kt][mq][e]);
       mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      const float m_new = fmaxf(m_i[mq], mx);
+      const float m_new = lazy_max(m_i[mq], mx);
       alpha[mq] = __builtin_amdgcn_exp2f((m_i[mq] - m_new) * SL2);
       m_i[mq] = m_new;
       const float msl = m_new * SL2;
@@ -405,7 +425,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
 #pragma unroll
         for (int e = 0; e < 16; ++e) mx = fmaxf(mx, s_acc[kt][mq][e]);
       mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      const float m_new = fmaxf(m_i[mq], mx);
+      const float m_new = lazy_max(m_i[mq], mx);
       alpha[mq] = __builtin_amdgcn_exp2f((m_i[mq] - m_new) * SL2);
       m_i[mq] = m_new;
       msl[mq] = m_new * SL2;
@@ -505,10 +525,10 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
   // One iteration = NS slots, one matrix instruction (per query tile) each: first
   // the S^T of tile j+1, then O^T += V_j^T P_j^T.  Every slot also carries a fixed
   // share of the vector work, so that the vector ALU runs in the shadow of the
-  // matrix pipe instead of in a phase of its own: the O^T rescale (S^T slots),
-  // the exponentials of tile j in three skewed stages (scale-and-shift in slot
-  // t-1, exp2 in slot t, row sum and fp16 packing in slot t+1; they run ahead of
-  // the O^T slots that consume them), and the running max of tile j+1 (O^T slots).
+  // matrix pipe instead of in a phase of its own: the exponentials of tile j in
+  // three skewed stages (scale-and-shift in slot t-1, exp2 in slot t, row sum and
+  // fp16 packing in slot t+1; they run ahead of the O^T slots that consume them),
+  // and the running max of tile j+1 (O^T slots).
   // Nothing moves across a slot boundary; operand fragments are read from LDS two
   // slots ahead.
   static_assert(STAGES == 2, "two K and two V slots");
@@ -516,7 +536,6 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
   constexpr int S_SLOTS = KT * DK, PV_SLOTS = KK * DT, NS = S_SLOTS + PV_SLOTS;
   constexpr int NE = KT * 16;             // scores per lane and query tile
   constexpr int NM = KT * 8;              // max3 operations of the running max
-  constexpr int NR = DT * 16;             // O^T registers to rescale
   constexpr int PVM = PV_SLOTS - 1;       // O^T slots that carry the running max
   struct Sched {
     static constexpr int ne_s() { return NE * 5 / 8; }          // exponentials under the S^T slots
@@ -542,7 +561,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
 #pragma unroll
     for (int mq = 0; mq < MQ; ++mq) {
       const float mxx = fmaxf(mx[mq], __shfl_xor(mx[mq], 32, 64));
-      const float m_new = fmaxf(m_i[mq], mxx);
+      const float m_new = lazy_max(m_i[mq], mxx);
       alpha[mq] = __builtin_amdgcn_exp2f((m_i[mq] - m_new) * SL2);
       m_i[mq] = m_new;
       msl[mq] = m_new * SL2;
@@ -606,13 +625,6 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
           constexpr int e = Sched::e_end(t) + decltype(ic)::value;
           sc[e / 16][mq][e % 16] = __builtin_fmaf(sc[e / 16][mq][e % 16], SL2, -msl[mq]);
         });
-        if constexpr (t >= 0 && t < S_SLOTS) {
-          constexpr int lo = (t * NR) / S_SLOTS, hi = ((t + 1) * NR) / S_SLOTS;
-          static_for<hi - lo>([&](auto ic) {
-            constexpr int i = lo + decltype(ic)::value;
-            o_acc[i / 16][mq][i % 16] *= alpha[mq];
-          });
-        }
         if constexpr (WITH_M && t >= S_SLOTS && t - S_SLOTS < PVM) {
           constexpr int u = t - S_SLOTS;
           if constexpr (u == 0) mx[mq] = sn[0][mq][0];
@@ -663,8 +675,9 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
     wait_and_barrier();  // K_{j+1}, V_j landed; everyone is done with K_j and V_{j-1}
     if (j + 2 < nkv) issue_k(j + 2, cur);
     issue_v(j + 1, cur ^ 1);
-    // (the rescale is unconditional here: a factor of 1 is exact, and a second copy of
-    // the slot sequence without it costs more registers than the skipped work is worth)
+    // The O^T rescale stays out of the slots: with the lazy running max it is needed
+    // for the first tile and then hardly ever, so it is a branch of its own here.
+    rescale_o();
 #if DECA_CAUSAL
     // One copy of the slot sequence only (a second one costs registers): the
     // running max stays out of the slots, and follows the mask.

@@ -136,6 +136,13 @@ def check_config(cfg: FAConfig, S_q: int, S_kv: int, D: int) -> None:
     assert est_regs_per_thread(cfg, D) <= 512
 
 
+# The kernel's running max follows a tile's max only when that lies more than this
+# many powers of two above it: p stays below 2^tau (fp16 P and fp32 sums hold that as
+# well as p <= 1), the quotient O / l is unchanged, and the O^T rescale is skipped for
+# almost every tile.
+LAZY_MAX_TAU = 8
+
+
 def make_flash_attn_fwd(
     B: int, H: int, S_q: int, S_kv: int, D: int, cfg: FAConfig,
     softmax_scale: float | None = None, causal: bool = False,
@@ -146,12 +153,13 @@ def make_flash_attn_fwd(
     check_config(cfg, S_q, S_kv, D)
     assert not causal or S_q == S_kv, "causal attention requires S_q == S_kv"
     scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(D)
+    assert scale > 0, "the running max is taken of the unscaled scores: the scale must be positive"
     defines = {
         "DECA_B": B, "DECA_H": H, "DECA_SQ": S_q, "DECA_SKV": S_kv, "DECA_D": D,
         "DECA_BR": cfg.Br, "DECA_BC": cfg.Bc, "DECA_NW": cfg.num_warps,
         "DECA_STAGES": cfg.stages, "DECA_CAUSAL": int(causal),
         "DECA_SCALE": repr(float(scale)), "DECA_PIPE": int(cfg.pipe),
-        "DECA_MIN_WAVES": target_waves_per_simd(cfg, D),
+        "DECA_MIN_WAVES": target_waves_per_simd(cfg, D), "DECA_LAZY_TAU": LAZY_MAX_TAU,
     }
     return make_spec(
         TEMPLATE, defines, grid=((S_q // cfg.Br) * B * H, 1, 1), block=(cfg.threads, 1, 1), nargs=4,

@@ -82,6 +82,33 @@ def test_flash_attn_large_scores():
     assert np.abs(got - oa.attention_f32(_f32(q), _f32(k), _f32(v), None, False)).max() <= 4e-3
 
 
+def _first_case(pipe, causal):
+    return next(c for c in FA_CASES if int(c[6].pipe) == pipe and c[5] == causal and c[2] == c[3] >= 512)
+
+
+@pytest.mark.parametrize("pipe", [0, 1, 2])
+@pytest.mark.parametrize("causal", [False, True])
+def test_flash_attn_growing_max(pipe, causal):
+    """Keys grow along the sequence, so the row maxima keep rising from tile to
+    tile: by less than the kernel's lazy-max threshold at first (stale max,
+    p > 1), then by more (rescale in the middle of the row)."""
+    from deca_amd.kernels.attn_bench import make_qkv_cpu
+
+    B, H, Sq, Skv, D, _, cfg = _first_case(pipe, causal)
+    print(f"case fa growing max B{B} H{H} S{Sq} D{D} causal={causal} {cfg}", flush=True)
+    q, k, v = make_qkv_cpu(B, H, Sq, Skv, D, seed=21)
+    ramp = torch.linspace(0.2, 6.0, Skv)[None, None, :, None]
+    k = (k.float() * ramp).half()
+    ref = oa.attention_f32(_f32(q), _f32(k), _f32(v), None, causal)
+    # the ramp does what it is for: per-tile maxima differ by more than 2^8 overall
+    s = np.einsum("bhqd,bhkd->bhqk", _f32(q), _f32(k)) * (1.4426950408889634 / np.sqrt(D))
+    tile_max = s.reshape(B, H, Sq, Skv // cfg.Bc, cfg.Bc).max(-1)
+    assert (tile_max.max(-1) - tile_max[..., 0]).max() > 16
+    got = _f32(_run(B, H, Sq, Skv, D, causal, cfg, q, k, v))
+    assert np.isfinite(got).all()
+    assert np.abs(got - ref).max() <= GATE
+
+
 @pytest.mark.parametrize("B,H,Sq,Skv,D,causal,cfg", FA_FULL, ids=lambda v: str(v))
 def test_flash_attn_full_size(B, H, Sq, Skv, D, causal, cfg):
     """Benchmark shapes: a few (batch, head) slices against the CPU checker,
