@@ -204,19 +204,19 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
   }
   // Inline assembly keeps the compiler's wait-count insertion from forcing
   // vmcnt(0) before every LDS read; waits are explicit and paired with barriers.
-  auto dma16 = [&](const _Float16* origin, unsigned voff, unsigned lds_addr) {
+  auto dma16 = [&](const _Float16* origin, unsigned voff, unsigned lds_addr) __attribute__((always_inline)) {
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                  :
                  : "v"(voff), "s"(origin), "s"(lds_addr)
                  : "memory");
   };
-  auto issue_k = [&](int j, int slot) {
+  auto issue_k = [&](int j, int slot) __attribute__((always_inline)) {
     const _Float16* origin = k_base + static_cast<size_t>(j) * BC * D_;
     const unsigned dst = lds_u + slot * TILE_BYTES + wave_u * 1024;
 #pragma unroll
     for (int it = 0; it < KV_IT; ++it) dma16(origin, k_voff[it], dst + it * NT * 16);
   };
-  auto issue_v = [&](int j, int slot) {
+  auto issue_v = [&](int j, int slot) __attribute__((always_inline)) {
     const _Float16* origin = v_base + static_cast<size_t>(j) * BC * D_;
     const unsigned dst = lds_u + (STAGES + slot) * TILE_BYTES + wave_u * 1024;
 #pragma unroll
@@ -267,7 +267,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
   static_assert(CPR >= 8, "D >= 64");
   // ---- the three phases of one KV step ----------------------------------------------------
   // S^T = K Q^T for the tile in K slot `kslot`
-  auto compute_s = [&](floatx16 (&s_acc)[KT][MQ], int kslot) {
+  auto compute_s = [&](floatx16 (&s_acc)[KT][MQ], int kslot) __attribute__((always_inline)) {
     const unsigned char* k_lds = lds + kslot * TILE_BYTES;
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt)
@@ -291,7 +291,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
   // Causal mask of tile j.  Only tiles crossing the diagonal need it; every
   // query sees key 0 in tile 0, so its running max is finite before a fully
   // masked block shows up.
-  auto mask_s = [&](floatx16 (&s_acc)[KT][MQ], int j) {
+  auto mask_s = [&](floatx16 (&s_acc)[KT][MQ], int j) __attribute__((always_inline)) {
 #if DECA_CAUSAL
     if ((j + 1) * BC - 1 > qt * BR + wave * WQ) {
 #pragma unroll
@@ -316,7 +316,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
   // then p = exp2((S - m) * sl2) stays below 2^DECA_LAZY_TAU, which fp16 P and
   // the fp32 sums hold as well as values below 1, and alpha is exactly 1, so
   // the O^T rescale is skipped.  O / l at the end is the same quotient.
-  auto lazy_max = [&](float m_old, float mx) {
+  auto lazy_max = [&](float m_old, float mx) __attribute__((always_inline)) {
     const float m_new = fmaxf(m_old, mx);
 #if DECA_LAZY_TAU > 0
     return (m_new - m_old) * SL2 > static_cast<float>(DECA_LAZY_TAU) ? m_new : m_old;
@@ -327,7 +327,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
   // Online softmax of one tile: one query column per lane.  Leaves P^T (fp16,
   // already in operand order) in `pf` and rescales O^T when a running max moved
   // (skipped otherwise: multiplying by 1 is exact).
-  auto softmax = [&](floatx16 (&s_acc)[KT][MQ], half8 (&pf)[KK][MQ]) {
+  auto softmax = [&](floatx16 (&s_acc)[KT][MQ], half8 (&pf)[KK][MQ]) __attribute__((always_inline)) {
     float alpha[MQ];
 #pragma unroll
     for (int mq = 0; mq < MQ; ++mq) {
@@ -375,7 +375,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
   // O^T += V^T P^T for the tile in V slot `vslot`.  k-slot (half, e) of step kk
   // is key row kk*16 + (e/4)*8 + half*4 + e%4: the order in which the S^T
   // accumulator registers hold the keys.
-  auto compute_pv = [&](const half8 (&pf)[KK][MQ], int vslot) {
+  auto compute_pv = [&](const half8 (&pf)[KK][MQ], int vslot) __attribute__((always_inline)) {
     const unsigned char* v_lds = lds + (STAGES + vslot) * TILE_BYTES;
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) {
@@ -397,7 +397,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
       }
     }
   };
-  auto wait_and_barrier = [&]() {
+  auto wait_and_barrier = [&]() __attribute__((always_inline)) {
     DECA_WAIT_VMCNT(0);                  // this lane's outstanding tile loads have landed
     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wave's LDS reads have returned
     __builtin_amdgcn_s_barrier();
@@ -416,7 +416,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
   static_assert(STAGES == 2, "the pipelined loop uses two K and two V slots");
   float alpha[MQ], msl[MQ];
   // m' = max(m, rowmax S); alpha = exp2((m - m') * sl2); msl = m' * sl2
-  auto row_stats = [&](const floatx16 (&s_acc)[KT][MQ]) {
+  auto row_stats = [&](const floatx16 (&s_acc)[KT][MQ]) __attribute__((always_inline)) {
 #pragma unroll
     for (int mq = 0; mq < MQ; ++mq) {
       float mx = s_acc[0][mq][0];
@@ -431,7 +431,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
       msl[mq] = m_new * SL2;
     }
   };
-  auto rescale_o = [&]() {
+  auto rescale_o = [&]() __attribute__((always_inline)) {
     bool moved = false;
 #pragma unroll
     for (int mq = 0; mq < MQ; ++mq) moved |= (alpha[mq] != 1.0f);
@@ -445,7 +445,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
     }
   };
   // p = exp2(S * sl2 - msl); l = l * alpha + sum p; P = fp16(p) in operand order
-  auto exp_and_pack = [&](floatx16 (&s_acc)[KT][MQ], half8 (&pf)[KK][MQ]) {
+  auto exp_and_pack = [&](floatx16 (&s_acc)[KT][MQ], half8 (&pf)[KK][MQ]) __attribute__((always_inline)) {
 #pragma unroll
     for (int mq = 0; mq < MQ; ++mq) {
       float sum = 0.0f;
@@ -557,7 +557,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
     }
   };
   static_assert(Sched::ok(), "the exponentials do not meet the O^T slots in time");
-  auto finish_stats = [&](float (&mx)[MQ]) {
+  auto finish_stats = [&](float (&mx)[MQ]) __attribute__((always_inline)) {
 #pragma unroll
     for (int mq = 0; mq < MQ; ++mq) {
       const float mxx = fmaxf(mx[mq], __shfl_xor(mx[mq], 32, 64));
@@ -568,7 +568,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
     }
   };
   half2v pf2[KK][MQ][4];
-  auto fused = [&](auto with_m, auto v_slot, floatx16 (&sc)[KT][MQ], floatx16 (&sn)[KT][MQ]) {
+  auto fused = [&](auto with_m, auto v_slot, floatx16 (&sc)[KT][MQ], floatx16 (&sn)[KT][MQ]) __attribute__((always_inline)) {
     constexpr bool WITH_M = decltype(with_m)::value;  // running max of tile j+1 in the O^T slots
     constexpr int VSLOT = decltype(v_slot)::value;  // V_j; K_{j+1} is in the other K slot
     const unsigned char* k_lds = lds + (VSLOT ^ 1) * TILE_BYTES;
@@ -576,7 +576,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
     const floatx16 zero = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f,
                            0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
     // slot t < S_SLOTS: pair p of key blocks, k-step ks, block kt; else k-step kk, d block dt
-    auto read_frag = [&](auto tc) -> half8 {
+    auto read_frag = [&](auto tc) __attribute__((always_inline)) -> half8 {
       constexpr int t = decltype(tc)::value;
       if constexpr (t < S_SLOTS) {
         constexpr int pr = t / (2 * DK), r = t % (2 * DK), ks = r / 2, kt = 2 * pr + r % 2;
@@ -600,10 +600,12 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
     // out of its slot, towards its first real use.
     auto pin = [](auto& v) { asm volatile("" : "+v"(v)); };
     // the vector work of slot t (t = -1: the scale-and-shift that slot 0 needs)
-    auto valu = [&](auto tc) {
+    auto valu = [&](auto tc) __attribute__((always_inline)) {
       constexpr int t = decltype(tc)::value;
-#pragma unroll
-      for (int mq = 0; mq < MQ; ++mq) {
+      // (compile-time loops over the query tiles: an unrolling pragma gives up on
+      // bodies of this size, and the accumulators would land in scratch memory)
+      static_for<MQ>([&](auto mqc) {
+        constexpr int mq = decltype(mqc)::value;
         // row sum and packing of what slot t-1 exponentiated
         static_for<Sched::e_end(t - 1) - Sched::e_end(t - 2)>([&](auto ic) {
           constexpr int e = Sched::e_end(t - 2) + decltype(ic)::value;
@@ -635,7 +637,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
             pin(mx[mq]);
           });
         }
-      }
+      });
     };
     half8 frag[3];
     frag[0] = read_frag(std::integral_constant<int, 0>{});
@@ -647,19 +649,20 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
       if constexpr (t + 2 < NS) frag[(t + 2) % 3] = read_frag(std::integral_constant<int, t + 2>{});
       if constexpr (t < S_SLOTS) {
         constexpr int pr = t / (2 * DK), r = t % (2 * DK), ks = r / 2, kt = 2 * pr + r % 2;
-#pragma unroll
-        for (int mq = 0; mq < MQ; ++mq)
+        static_for<MQ>([&](auto mqc) {
+          constexpr int mq = decltype(mqc)::value;
           sn[kt][mq] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
               frag[t % 3], qf[mq][ks], ks == 0 ? zero : sn[kt][mq], 0, 0, 0);
+        });
       } else {
         constexpr int u = t - S_SLOTS, kk = u / DT, dt = u % DT;
-#pragma unroll
-        for (int mq = 0; mq < MQ; ++mq) {
+        static_for<MQ>([&](auto mqc) {
+          constexpr int mq = decltype(mqc)::value;
           const half8 pfr = __builtin_shufflevector(
               __builtin_shufflevector(pf2[kk][mq][0], pf2[kk][mq][1], 0, 1, 2, 3),
               __builtin_shufflevector(pf2[kk][mq][2], pf2[kk][mq][3], 0, 1, 2, 3), 0, 1, 2, 3, 4, 5, 6, 7);
           o_acc[dt][mq] = __builtin_amdgcn_mfma_f32_32x32x16_f16(frag[t % 3], pfr, o_acc[dt][mq], 0, 0, 0);
-        }
+        });
       }
       valu(tc);
       __builtin_amdgcn_sched_barrier(0);
@@ -670,7 +673,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
   };
   half8 pf[KK][MQ];
   // tile j: softmax and second product; tile j+1: first product and row statistics
-  auto step = [&](auto cur_slot, floatx16 (&sc)[KT][MQ], floatx16 (&sn)[KT][MQ], int j) {
+  auto step = [&](auto cur_slot, floatx16 (&sc)[KT][MQ], floatx16 (&sn)[KT][MQ], int j) __attribute__((always_inline)) {
     constexpr int cur = decltype(cur_slot)::value;  // == j % 2
     wait_and_barrier();  // K_{j+1}, V_j landed; everyone is done with K_j and V_{j-1}
     if (j + 2 < nkv) issue_k(j + 2, cur);
@@ -688,7 +691,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
     fused(std::integral_constant<bool, true>{}, cur_slot, sc, sn);
 #endif
   };
-  auto tail = [&](floatx16 (&sc)[KT][MQ], int j) {
+  auto tail = [&](floatx16 (&sc)[KT][MQ], int j) __attribute__((always_inline)) {
     wait_and_barrier();
 #if DECA_CAUSAL
     // every key of the last tile lies after every query row of this wave: P = 0 exactly
