@@ -377,7 +377,7 @@ FA_DOMAINS = {
 
 def _fa_constraints(arch, B: int, H: int, S_q: int, S_kv: int, D: int, type_size: int,
                     max_est_regs: int):
-    from deca_amd.kernels.flash_attn_hip import slot_schedule_ok
+    from deca_amd.kernels.flash_attn_hip import SPILL_FREE_EST_REGS, slot_schedule_ok
 
     wave = arch.warp_size
     simds = arch.simds_per_cu
@@ -419,6 +419,9 @@ def _fa_constraints(arch, B: int, H: int, S_q: int, S_kv: int, D: int, type_size
         regs8 = o.udiv(regs + 7, c(8)) * 8
         waves_per_simd = o.udiv(nw + (simds - 1), c(simds))
         out += [o.ule(regs, c(max_est_regs)), o.ule(regs8 * waves_per_simd, c(arch.vgprs_per_simd))]
+        # what the compiler was seen to allocate without spilling, per loop shape
+        for (p_, st_), limit in SPILL_FREE_EST_REGS.items():
+            out.append(o.implies(o.all_of(o.eq(pipe, c(p_)), o.eq(st, c(st_))), o.ule(regs, c(limit))))
         # enough workgroups to give every CU at least one
         out.append(o.uge(o.udiv(c(S_q), br) * (B * H), c(arch.sm_nums)))
         return out

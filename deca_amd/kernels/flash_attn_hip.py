@@ -81,6 +81,21 @@ def est_regs_per_thread(cfg: FAConfig, D: int) -> int:
     return o_acc + s_acc + p_h + q_frag + kv_frag + 4 * mq + 40
 
 
+# Largest register estimate that hipcc was seen to allocate without spilling, by
+# (pipe, stages).  A wave that is alone on its SIMD may use all 512 registers, and the
+# compiler then spends them on scheduling freedom: measured allocations are 1.35-1.4x the
+# estimate for the plain loop with one LDS stage, 1.5x and more with two (the two unrolled
+# steps overlap), 1.0-1.3x for the loops whose order is fixed by hand.  Beyond these the
+# kernels spill to scratch memory inside the loop and run 2-15x slower.
+SPILL_FREE_EST_REGS = {(0, 1): 365, (0, 2): 330, (1, 2): 480, (2, 2): 480}
+
+
+def expect_spill_free(cfg: FAConfig, D: int) -> bool:
+    """Whether the compiler is expected to fit the kernel's registers (see above)."""
+    limit = SPILL_FREE_EST_REGS.get((int(cfg.pipe), cfg.stages))
+    return limit is not None and est_regs_per_thread(cfg, D) <= limit
+
+
 def target_waves_per_simd(cfg: FAConfig, D: int) -> int:
     """Waves per SIMD the kernel is compiled for: what the estimated registers and the LDS
     footprint let co-reside.  Without it the compiler spends the whole 512-register file on

@@ -146,7 +146,7 @@ def test_flash_attn_configs_are_valid(D, S):
         if (S // br) * B * H < ARCH.sm_nums or st > S // bc or (pipe and S // bc < 2):
             continue
         regs = (fa.est_regs_per_thread(cfg, D) + 7) // 8 * 8
-        if regs * -(-nw // 4) > 512:
+        if regs * -(-nw // 4) > 512 or not fa.expect_spill_free(cfg, D):
             continue
         want.add(cfg)
     assert set(configs) == want
@@ -154,6 +154,27 @@ def test_flash_attn_configs_are_valid(D, S):
     tight = Solver.solve_flash_attn(ARCH, B, H, S, S, D, max_est_regs=256)
     assert set(tight) < set(configs) or set(tight) == set(configs)
     assert all(fa.est_regs_per_thread(c, D) <= 256 for c in tight)
+
+
+def test_flash_attn_register_limits_follow_the_compiler():
+    """The per-loop-shape limits on the register estimate: just below them hipcc
+    allocates without spilling, the first estimate above them spills."""
+    from deca_amd.kernels.build import kernel_resources
+
+    def resources(cfg, D):
+        return kernel_resources(fa.make_flash_attn_fwd(4, 16, 4096, 4096, D, cfg, None, False))
+
+    keep = fa.FAConfig(256, 64, 4, 1)   # D = 128: estimate 352 <= 365, one LDS stage
+    drop = fa.FAConfig(256, 64, 4, 2)   # same tile, two stages: limit 330
+    assert fa.expect_spill_free(keep, 128) and not fa.expect_spill_free(drop, 128)
+    configs = Solver.solve_flash_attn(ARCH, 4, 16, 4096, 4096, 128)
+    assert keep in configs and drop not in configs
+    assert resources(keep, 128)["vgpr_spills"] == 0
+    assert resources(drop, 128)["vgpr_spills"] > 0
+    slots = fa.FAConfig(256, 64, 4, 2, pipe=2)  # estimate 384 <= 480
+    assert slots in configs
+    got = resources(slots, 128)
+    assert got["vgpr_spills"] == 0 and got["scratch_bytes"] == 0
 
 
 def test_z3_backend_agrees_with_enumeration():
