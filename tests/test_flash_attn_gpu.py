@@ -44,6 +44,11 @@ def test_flash_attn_parity(B, H, Sq, Skv, D, causal, cfg):
     assert np.abs(got - ref).max() <= GATE
     tiled = oa.flash_blockwise(_f32(q), _f32(k), _f32(v), None, causal, cfg.Br, cfg.Bc)
     assert np.abs(got - tiled).max() <= GATE
+    # and of the same recurrence with the kernel's lazy running max
+    from deca_amd.kernels.flash_attn_hip import LAZY_MAX_TAU
+
+    lazy = oa.flash_blockwise(_f32(q), _f32(k), _f32(v), None, causal, cfg.Br, cfg.Bc, lazy_tau=LAZY_MAX_TAU)
+    assert np.abs(got - lazy).max() <= GATE
 
 
 def test_flash_attn_closed_forms():

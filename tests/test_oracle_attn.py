@@ -52,6 +52,29 @@ def test_blockwise_matches_plain_and_tiling_does_not_matter(causal):
     assert np.abs(one - many).max() < 2e-3
 
 
+@pytest.mark.parametrize("causal", [False, True])
+def test_lazy_running_max_is_the_same_quotient(causal):
+    """The kernel's lazy running max against the reference's eager one: keys grow
+    along the sequence, so that rows stay below the threshold for some tiles
+    (stale max, p > 1) and cross it at others."""
+    q, k, v = _qkv(1, 2, 256, 256, 64, seed=4)
+    k = k * np.linspace(0.2, 6.0, 256, dtype=np.float32)[None, None, :, None]
+    k = k.astype(np.float16).astype(np.float32)
+    ref = oa.attention_f32(q, k, v, None, causal)
+    eager = oa.flash_blockwise(q, k, v, None, causal, Br=64, Bc=32)
+    lazy = oa.flash_blockwise(q, k, v, None, causal, Br=64, Bc=32, lazy_tau=8.0)
+    assert np.abs(eager - ref).max() < 2e-3 and np.abs(lazy - ref).max() < 2e-3
+    assert np.abs(lazy - eager).max() < 2e-3
+    # the two recurrences did take different paths: count the tiles that move a max
+    sl2 = 1.4426950408889634 / 8.0
+    s = np.einsum("bhqd,bhkd->bhqk", q, k) * sl2
+    if causal:
+        s = np.where(np.arange(256)[None, :] > np.arange(256)[:, None], -np.inf, s)
+    run = np.maximum.accumulate(s.reshape(1, 2, 256, 8, 32).max(-1), axis=-1)
+    steps = np.diff(run, axis=-1)
+    assert (steps > 0).sum() > 2 * ((steps > 8).sum() + 1)
+
+
 def test_cross_attention_lengths_and_scale():
     q, k, v = _qkv(2, 1, 64, 192, 128, seed=3)
     ref = oa.attention_f32(q, k, v, 0.05, False)
