@@ -268,7 +268,7 @@ GEMM_RASTERS = (0, 1, 2, 4, 8, 16)  # 0: 8 x 4 sub-blocks of tiles per XCD, neig
 
 
 def _gemm_constraints(arch, M: int, N: int, K: int, type_size: int):
-    from deca_amd.kernels.gemm_hip import EPI_PAD
+    from deca_amd.kernels.gemm_hip import EPI_PAD, SPILL_FREE_EST_REGS
 
     wave = arch.warp_size
     simds = arch.simds_per_cu
@@ -309,7 +309,7 @@ def _gemm_constraints(arch, M: int, N: int, K: int, type_size: int):
         regs = acc + 2 * frags + staging + 40
         regs8 = o.udiv(regs + 7, c(8)) * 8
         waves_per_simd = o.udiv(waves + (simds - 1), c(simds))
-        out += [o.ule(regs, c(arch.vgprs_per_simd)),
+        out += [o.ule(regs, c(min(arch.vgprs_per_simd, SPILL_FREE_EST_REGS))),
                 o.ule(regs8 * waves_per_simd, c(arch.vgprs_per_simd))]
         # the loads of the (st - 2) youngest tiles stay in flight across a wait: the
         # vector-memory counter holds 6 bits

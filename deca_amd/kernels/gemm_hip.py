@@ -90,6 +90,12 @@ def smem_bytes(cfg: GemmConfig) -> int:
     return max(pipeline_smem_bytes(cfg), epilogue_smem_bytes(cfg))
 
 
+# Largest register estimate hipcc was seen to allocate without spilling: the estimate
+# tracks the compiler's allocation within a few registers up to here; the tile sets
+# above it (128 x 128 wave tiles staged through registers) spill in the main loop.
+SPILL_FREE_EST_REGS = 456
+
+
 def est_regs_per_thread(cfg: GemmConfig) -> int:
     """Unified VGPR estimate per lane: fp32 accumulators (warp_m * warp_n / 64),
     one set of A / B fragments (4 VGPRs per 32-row tile), the global->LDS

@@ -103,7 +103,7 @@ def test_gemm_configs_are_valid(n):
         if (n // bm) * (n // bn) < ARCH.sm_nums:
             continue
         regs = (gm.est_regs_per_thread(cfg) + 7) // 8 * 8
-        if regs * -(-cfg.num_warps // 4) > 512:
+        if regs * -(-cfg.num_warps // 4) > 512 or gm.est_regs_per_thread(cfg) > gm.SPILL_FREE_EST_REGS:
             continue
         tiles.add((bm, bn, bk, wm, wn, st, epi, direct))
     got = {(c.BM, c.BN, c.BK, c.warp_m, c.warp_n, c.stages, c.epi_smem, c.direct) for c in configs}
