@@ -403,6 +403,34 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
     __builtin_amdgcn_s_barrier();
   };
 
+#if STAGES == 2
+  // One KV step.  `slot` is a literal at both call sites, so that every LDS
+  // address of the step is "lane base + immediate" and needs no address arithmetic.
+  auto kv_step = [&](int j, int slot) __attribute__((always_inline)) {
+    // Tile j has landed for every lane, and every wave is done with the slot
+    // that tile j+1 is about to overwrite.
+    wait_and_barrier();
+    if (j + 1 < nkv) {
+      issue_k(j + 1, slot ^ 1);
+      issue_v(j + 1, slot ^ 1);
+    }
+#if DECA_CAUSAL
+    // Every key of the tile lies after every query row of this wave (the last tile
+    // of a workgroup with BR > BC): all its scores are masked, P = 0 exactly, and
+    // there is nothing to add.  (Skipping single masked 32-key blocks of the
+    // diagonal tiles as well was tried: the extra code paths cost registers and
+    // made the kernel slower.)
+    if (j * BC > qt * BR + wave_u * WQ + WQ - 1) return;
+#endif
+    floatx16 s_acc[KT][MQ];
+    half8 pf[KK][MQ];
+    compute_s(s_acc, slot);
+    mask_s(s_acc, j);
+    softmax(s_acc, pf);
+    compute_pv(pf, slot);
+  };
+#endif
+
 #if DECA_PIPE
   // ---- software-pipelined loop ------------------------------------------------------------
   // S^T of tile j+1 is computed in the same straight-line block as the
@@ -568,8 +596,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
     }
   };
   half2v pf2[KK][MQ][4];
-  auto fused = [&](auto with_m, auto v_slot, floatx16 (&sc)[KT][MQ], floatx16 (&sn)[KT][MQ]) __attribute__((always_inline)) {
-    constexpr bool WITH_M = decltype(with_m)::value;  // running max of tile j+1 in the O^T slots
+  auto fused = [&](auto v_slot, floatx16 (&sc)[KT][MQ], floatx16 (&sn)[KT][MQ]) __attribute__((always_inline)) {
     constexpr int VSLOT = decltype(v_slot)::value;  // V_j; K_{j+1} is in the other K slot
     const unsigned char* k_lds = lds + (VSLOT ^ 1) * TILE_BYTES;
     const unsigned char* v_lds = lds + (STAGES + VSLOT) * TILE_BYTES;
@@ -627,7 +654,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
           constexpr int e = Sched::e_end(t) + decltype(ic)::value;
           sc[e / 16][mq][e % 16] = __builtin_fmaf(sc[e / 16][mq][e % 16], SL2, -msl[mq]);
         });
-        if constexpr (WITH_M && t >= S_SLOTS && t - S_SLOTS < PVM) {
+        if constexpr (t >= S_SLOTS && t - S_SLOTS < PVM) {
           constexpr int u = t - S_SLOTS;
           if constexpr (u == 0) mx[mq] = sn[0][mq][0];
           constexpr int lo = (u * NM) / PVM, hi = ((u + 1) * NM) / PVM;
@@ -669,7 +696,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
     });
 #pragma unroll
     for (int mq = 0; mq < MQ; ++mq) l_i[mq] = l_i[mq] * alpha[mq] + (sum[mq][0] + sum[mq][1]);
-    if (WITH_M) finish_stats(mx);
+    finish_stats(mx);
   };
   half8 pf[KK][MQ];
   // tile j: softmax and second product; tile j+1: first product and row statistics
@@ -681,38 +708,67 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
     // The O^T rescale stays out of the slots: with the lazy running max it is needed
     // for the first tile and then hardly ever, so it is a branch of its own here.
     rescale_o();
-#if DECA_CAUSAL
-    // One copy of the slot sequence only (a second one costs registers): the
-    // running max stays out of the slots, and follows the mask.
-    fused(std::integral_constant<bool, false>{}, cur_slot, sc, sn);
-    mask_s(sn, j + 1);
-    row_stats(sn);
-#else
-    fused(std::integral_constant<bool, true>{}, cur_slot, sc, sn);
-#endif
+    fused(cur_slot, sc, sn);
   };
   auto tail = [&](floatx16 (&sc)[KT][MQ], int j) __attribute__((always_inline)) {
     wait_and_barrier();
 #if DECA_CAUSAL
-    // every key of the last tile lies after every query row of this wave: P = 0 exactly
-    if (j * BC > qt * BR + wave_u * WQ + WQ - 1) return;
+    // the diagonal tiles follow: V_{j+1} goes where V_{j-1} was (K_{j+1} is under way)
+    issue_v(j + 1, (j + 1) & 1);
 #endif
     rescale_o();
     exp_and_pack(sc, pf);
     compute_pv(pf, j & 1);
   };
+  const std::integral_constant<int, 0> even;
+  const std::integral_constant<int, 1> odd;
+#if DECA_CAUSAL
+  // Two phases.  The nd tiles that lie below the diagonal for every row of the
+  // workgroup need no mask: they run through the slot loop.  The tiles that reach
+  // the diagonal follow as plain steps (S^T, mask, softmax, O^T one after the
+  // other), which keeps a second, mask-aware copy of the slot sequence out of the
+  // register allocation.
+  const int nd = (qt * BR) / BC;
+  int j0 = 0;
+  issue_k(0, 0);
+  issue_v(0, 0);
+  if (nd >= 2) {
+    issue_k(1, 1);
+    floatx16 s_a[KT][MQ], s_b[KT][MQ];
+    wait_and_barrier();
+    compute_s(s_a, 0);
+    row_stats(s_a);
+    int j = 0;
+    for (; j + 2 < nd; j += 2) {
+      step(even, s_a, s_b, j);
+      step(odd, s_b, s_a, j + 1);
+    }
+    if (j + 1 < nd) {
+      step(even, s_a, s_b, j);
+      tail(s_b, j + 1);
+    } else {
+      tail(s_a, j);
+    }
+    j0 = nd;
+  }
+  if (j0 & 1) {
+    kv_step(j0, 1);
+    ++j0;
+  }
+  for (int j = j0; j < nkv; j += 2) {
+    kv_step(j, 0);
+    if (j + 1 < nkv) kv_step(j + 1, 1);
+  }
+#else
   issue_k(0, 0);
   issue_v(0, 0);
   if (nkv > 1) issue_k(1, 1);
   floatx16 s_a[KT][MQ], s_b[KT][MQ];
   wait_and_barrier();
   compute_s(s_a, 0);
-  mask_s(s_a, 0);
   row_stats(s_a);
   {
     int j = 0;
-    const std::integral_constant<int, 0> even;
-    const std::integral_constant<int, 1> odd;
     for (; j + 2 < nkv; j += 2) {
       step(even, s_a, s_b, j);
       step(odd, s_b, s_a, j + 1);
@@ -724,6 +780,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
       tail(s_a, j);
     }
   }
+#endif
 #else
   issue_k(0, 0);
   issue_v(0, 0);
@@ -766,31 +823,6 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
   issue_k(0, 0);
   issue_v(0, 0);
 #if STAGES == 2
-  // One KV step.  `slot` is a literal at both call sites, so that every LDS
-  // address of the step is "lane base + immediate" and needs no address arithmetic.
-  auto kv_step = [&](int j, int slot) __attribute__((always_inline)) {
-    // Tile j has landed for every lane, and every wave is done with the slot
-    // that tile j+1 is about to overwrite.
-    wait_and_barrier();
-    if (j + 1 < nkv) {
-      issue_k(j + 1, slot ^ 1);
-      issue_v(j + 1, slot ^ 1);
-    }
-#if DECA_CAUSAL
-    // Every key of the tile lies after every query row of this wave (the last tile
-    // of a workgroup with BR > BC): all its scores are masked, P = 0 exactly, and
-    // there is nothing to add.  (Skipping single masked 32-key blocks of the
-    // diagonal tiles as well was tried: the extra code paths cost registers and
-    // made the kernel slower.)
-    if (j * BC > qt * BR + wave_u * WQ + WQ - 1) return;
-#endif
-    floatx16 s_acc[KT][MQ];
-    half8 pf[KK][MQ];
-    compute_s(s_acc, slot);
-    mask_s(s_acc, j);
-    softmax(s_acc, pf);
-    compute_pv(pf, slot);
-  };
   for (int j = 0; j < nkv; j += 2) {
     kv_step(j, 0);
     if (j + 1 < nkv) kv_step(j + 1, 1);
