@@ -148,6 +148,10 @@ FA_CASES = [
     (1, 2, 128, 192, 64, False, FAConfig(128, 64, 2, 2, pipe=2)),    # two query tiles per wave
     (1, 1, 128, 64, 64, False, FAConfig(64, 64, 2, 2, pipe=2)),      # a single KV tile
     (1, 1, 128, 128, 64, True, FAConfig(64, 64, 2, 2, pipe=2)),      # two KV tiles, no loop
+    # causal slot loop: an odd number of unmasked tiles ahead of the diagonal ones, and
+    # key tiles wider than the query tiles
+    (1, 2, 512, 512, 64, True, FAConfig(128, 128, 4, 2, pipe=2)),
+    (1, 2, 1024, 1024, 64, True, FAConfig(64, 128, 2, 2, pipe=2)),
 ]
 
 FA_FULL = [
@@ -157,6 +161,8 @@ FA_FULL = [
     (4, 16, 4096, 4096, 64, True, FAConfig(128, 64, 4, 2)),
     (4, 16, 4096, 4096, 128, True, FAConfig(256, 128, 8, 2)),
     (4, 16, 4096, 4096, 64, False, FAConfig(256, 128, 8, 2, pipe=2)),
+    (4, 16, 4096, 4096, 128, False, FAConfig(256, 64, 8, 2, pipe=2)),
+    (4, 16, 4096, 4096, 128, True, FAConfig(256, 64, 8, 2, pipe=2)),
 ]
 
 
