@@ -316,15 +316,29 @@ def fa_score(cfg, arch, shape, causal: bool = False) -> float:
     t_flop = max(t_flop, t_valu)
 
     pipe = 1.0 if cfg.stages >= 2 else 0.96
+    # S^T one tile ahead without the slots: two S^T accumulators and a longer dependent
+    # chain for nothing in return (measured 2-8 % behind the plain loop of the same tile)
+    if int(cfg.pipe) == 1:
+        pipe *= 0.95
     sync = 1.0 / (1.0 + getattr(arch, "fa_cta_sync_penalty", 0.0) * cfg.num_warps / 4 / wgs)
-    # longer KV steps amortise the per-step max / rescale / barrier
-    step = 1.0 / (1.0 + 0.06 * 64 / cfg.Bc)
+    # longer KV steps amortise the per-step max / barrier; the slot loop has the row
+    # statistics inside the matrix work and pays a third of it
+    step = 1.0 / (1.0 + (0.02 if int(cfg.pipe) == 2 else 0.06) * 64 / cfg.Bc)
 
     useful = 1.0
     if causal:
+        # a wave computes every tile that reaches one of its rows in full and skips the
+        # tiles beyond its last row
         nq = S_q // cfg.Br
-        computed = sum(-(-(i + 1) * cfg.Br // cfg.Bc) * cfg.Bc for i in range(nq)) * cfg.Br
+        computed = sum(-(-(i * cfg.Br + (w + 1) * wq) // cfg.Bc) * cfg.Bc * wq
+                       for i in range(nq) for w in range(cfg.num_warps))
         useful = S_q * (S_q + 1) / 2 / computed
+        # The workgroups of a causal launch differ in length, and towards the end many CUs
+        # hold a single one.  A workgroup that fills its SIMDs with two waves by itself keeps
+        # its overlap partner until the end; a smaller one does not (measured: the causal /
+        # full ratio of 4-wave configs is 0.84-0.86, of 8-wave configs 0.90).
+        if cfg.num_warps < 2 * arch.simds_per_cu:
+            useful *= 0.94
 
     # every further 32-query tile of a wave lengthens the dependent chain between barriers
     chain = 1.0 / (1.0 + 0.05 * (wq // 32 - 1))

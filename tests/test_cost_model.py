@@ -88,11 +88,12 @@ def test_fa_score_terms():
     assert s > 0
     assert cm.fa_score(FAConfig(256, 128, 8, 1), ARCH, shape) < s       # single slot exposes latency
     assert cm.fa_score(a, ARCH, shape, causal=True) < s                  # diagonal tiles are wasted work
-    # causal useful fraction: Br = Bc = S means one tile, half of it useful
+    # causal useful fraction: a wave computes the tiles that reach its 32 rows in full
     one = FAConfig(256, 128, 8, 1)
     nq, computed = 4096 // 256, 0
     for i in range(nq):
-        computed += math.ceil((i + 1) * 256 / 128) * 128 * 256
+        for w in range(8):
+            computed += math.ceil((i * 256 + (w + 1) * 32) / 128) * 128 * 32
     ratio = cm.fa_score(one, ARCH, shape, True) / cm.fa_score(one, ARCH, shape, False)
     # ... times the start-up latency of a workgroup, which weighs more on the halved KV loop
     rate = 0.42 * ARCH.peak_mma_sync_flops * 1e9 / ARCH.sm_nums
@@ -103,6 +104,14 @@ def test_fa_score_terms():
     short = (32, 16, 512, 512, 128)
     assert (cm.fa_score(FAConfig(128, 64, 4, 2), ARCH, short) / cm.fa_score(a, ARCH, short)
             > cm.fa_score(FAConfig(128, 64, 4, 2), ARCH, shape) / cm.fa_score(a, ARCH, shape))
+    # the loop shapes: S^T one tile ahead without the slots trails the plain loop, the slot
+    # loop leads it; a causal launch costs the small workgroups their overlap partner
+    b = FAConfig(256, 64, 8, 2)
+    assert (cm.fa_score(FAConfig(256, 64, 8, 2, pipe=1), ARCH, shape) < cm.fa_score(b, ARCH, shape)
+            < cm.fa_score(FAConfig(256, 64, 8, 2, pipe=2), ARCH, shape))
+    small = FAConfig(128, 64, 4, 2)
+    assert (cm.fa_score(small, ARCH, shape, True) / cm.fa_score(small, ARCH, shape)
+            < cm.fa_score(b, ARCH, shape, True) / cm.fa_score(b, ARCH, shape))
     wgs, share = cm.fa_occupancy(a, ARCH, 128, 1024)
     assert wgs == 1 and share == pytest.approx(8 / 32)
     assert cm.rank_fa_configs([FAConfig(32, 32, 1, 1), a], ARCH, shape, top_n=1) == [a]
