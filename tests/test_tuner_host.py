@@ -208,6 +208,27 @@ def test_tuned_table_roundtrip(tmp_path):
     assert len(bench.workloads()) == 13
 
 
+def test_shipped_winners_are_solver_candidates():
+    """Every entry of the shipped table is a configuration its solver still emits for
+    that shape (a rule added to a solver must not leave a stale winner behind)."""
+    from deca_amd import Solver, tuned
+    from deca_amd.arch import MI355X
+
+    arch = MI355X()
+    table = tuned.load()
+    assert table
+    for key in table:
+        op, dims = key.split("|")[0], tuple(int(d) for d in key.split("|")[1].split("x"))
+        cfg = tuned.lookup(key)
+        if op == "GEMM":
+            candidates = Solver.solve_gemm_tc(arch, *dims)
+        elif op == "flash_attn":
+            candidates = Solver.solve_flash_attn(arch, *dims)
+        else:
+            candidates = Solver.solve_rowwise(arch, op, *dims)
+        assert cfg in candidates, key
+
+
 def test_rotating_sets_and_cycle():
     import torch
 
