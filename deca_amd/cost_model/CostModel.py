@@ -319,11 +319,11 @@ def fa_score(cfg, arch, shape, causal: bool = False) -> float:
     # S^T one tile ahead without the slots: two S^T accumulators and a longer dependent
     # chain for nothing in return (measured 2-8 % behind the plain loop of the same tile)
     if int(cfg.pipe) == 1:
-        pipe *= 0.95
+        pipe *= 0.90
     sync = 1.0 / (1.0 + getattr(arch, "fa_cta_sync_penalty", 0.0) * cfg.num_warps / 4 / wgs)
     # longer KV steps amortise the per-step max / barrier; the slot loop has the row
-    # statistics inside the matrix work and pays a third of it
-    step = 1.0 / (1.0 + (0.02 if int(cfg.pipe) == 2 else 0.06) * 64 / cfg.Bc)
+    # statistics inside the matrix work and pays a little less of it
+    step = 1.0 / (1.0 + (0.06 if int(cfg.pipe) == 2 else 0.08) * 64 / cfg.Bc)
 
     useful = 1.0
     if causal:
@@ -338,19 +338,23 @@ def fa_score(cfg, arch, shape, causal: bool = False) -> float:
         # its overlap partner until the end; a smaller one does not (measured: the causal /
         # full ratio of 4-wave configs is 0.84-0.86, of 8-wave configs 0.90).
         if cfg.num_warps < 2 * arch.simds_per_cu:
-            useful *= 0.94
+            useful *= 0.90
+        # and a wave with more than one 32-query tile skips fewer masked tiles
+        useful /= 1.0 + 0.09 * (wq // 32 - 1)
 
     # every further 32-query tile of a wave lengthens the dependent chain between barriers
-    chain = 1.0 / (1.0 + 0.05 * (wq // 32 - 1))
+    chain = 1.0 / (1.0 + 0.20 * (wq // 32 - 1))
 
     # A workgroup starts with nothing in flight (Q, then the first K/V tile) and ends with
     # the O store: a few microseconds that only another resident workgroup can cover.
     # It matters when the KV loop is short (measured at S = 512: two 4-wave workgroups per
-    # CU beat one 8-wave workgroup by 20 %).  The constants are a compromise between that
-    # shape and S = 4096, D = 64, where a stronger term would rank 4-wave configs too high.
+    # CU beat one 8-wave workgroup by 20 %).  This and the other constants of this function
+    # were fitted on exhaustive measurements of twelve shapes (S = 512, 1024, 4096; D = 64,
+    # 128; full and causal): the measured best is then among the first 8 for all of them
+    # and among the first 3 for ten.
     kv_len = S_kv * (0.5 if causal else 1.0)
     t_loop = 4.0 * cfg.Br * kv_len * D / (0.42 * arch.peak_mma_sync_flops * 1e9 / cus)
-    exposed = getattr(arch, "fa_workgroup_latency_s", 2e-6) * (1.0 if wgs == 1 else _FA_HIDDEN)
+    exposed = getattr(arch, "fa_workgroup_latency_s", 4e-6) * (1.0 if wgs == 1 else _FA_HIDDEN)
     ramp = t_loop / (t_loop + exposed)
 
     return wave_eff * pipe * sync * step * useful * chain * ramp / (t_flop / t_mma)

@@ -97,7 +97,7 @@ def test_fa_score_terms():
     ratio = cm.fa_score(one, ARCH, shape, True) / cm.fa_score(one, ARCH, shape, False)
     # ... times the start-up latency of a workgroup, which weighs more on the halved KV loop
     rate = 0.42 * ARCH.peak_mma_sync_flops * 1e9 / ARCH.sm_nums
-    t_full, lat = 4.0 * 256 * 4096 * 128 / rate, 2e-6
+    t_full, lat = 4.0 * 256 * 4096 * 128 / rate, 4e-6
     ramp = (t_full / 2 / (t_full / 2 + lat)) / (t_full / (t_full + lat))
     assert ratio == pytest.approx(4096 * 4097 / 2 / computed * ramp)
     # a short KV loop favours two resident workgroups over one that owns the CU
