@@ -340,10 +340,11 @@ def fa_score(cfg, arch, shape, causal: bool = False) -> float:
         if cfg.num_warps < 2 * arch.simds_per_cu:
             useful *= 0.90
         # and a wave with more than one 32-query tile skips fewer masked tiles
-        useful /= 1.0 + 0.09 * (wq // 32 - 1)
+        useful /= 1.0 + 0.15 * (wq // 32 - 1)
 
     # every further 32-query tile of a wave lengthens the dependent chain between barriers
-    chain = 1.0 / (1.0 + 0.20 * (wq // 32 - 1))
+    # and the prologue (twice the Q fragments): 17 % at S = 512, 2 % on long sequences
+    chain = 1.0 / (1.0 + (0.02 + 0.18 * min(1.0, 512.0 / S_kv)) * (wq // 32 - 1))
 
     # A workgroup starts with nothing in flight (Q, then the first K/V tile) and ends with
     # the O store: a few microseconds that only another resident workgroup can cover.
