@@ -118,9 +118,15 @@ class _Z3Ops:  # pragma: no cover - exercised only when z3 is installed
 def _enumerate(domains: dict, constraints, count: int, backend: str = "auto"):
     """All assignments of `domains` (name -> tuple of ints) that satisfy
     `constraints(ops, vars) -> list of boolean expressions`, as sorted tuples in
-    the key order of `domains`, at most `count` of them."""
+    the key order of `domains`, at most `count` of them.
+
+    `backend`: "enum" (and "auto") walk the finite domains exhaustively; "z3"
+    runs the same constraints through a Z3 all-SAT loop with blocking clauses,
+    as the reference does (Solver.py:543-558).  The Z3 path is only taken when
+    it is asked for by name: no environment this package was developed in has
+    z3, so that path has never been executed."""
     names = list(domains)
-    use_z3 = backend == "z3" or (backend == "auto" and _z3 is not None)
+    use_z3 = backend == "z3"
     if use_z3:
         if _z3 is None:
             raise RuntimeError("z3 backend requested but z3 is not importable")
@@ -260,9 +266,10 @@ GEMM_DOMAINS = {
     "bk": (32, 64),
     "wm": (32, 64, 128),
     "wn": (32, 64, 128),
-    "st": (1, 2, 3, 4),
+    "st": (1, 2, 3, 4, 5),
     "epi": (0, 1),
     "direct": (0, 1),
+    "mfma": (32, 16),  # 32: v_mfma_f32_32x32x16, 16: v_mfma_f32_16x16x32
 }
 GEMM_RASTERS = (0, 1, 2, 4, 8, 16)  # 0: 8 x 4 sub-blocks of tiles per XCD, neighbours in flight
 
@@ -274,7 +281,7 @@ def _gemm_constraints(arch, M: int, N: int, K: int, type_size: int):
     simds = arch.simds_per_cu
 
     def build(o, v):
-        bm, bn, bk, wm, wn, st, epi, direct = (v[k] for k in GEMM_DOMAINS)
+        bm, bn, bk, wm, wn, st, epi, direct, mfma = (v[k] for k in GEMM_DOMAINS)
         c = o.const
         m_, n_, k_ = c(M), c(N), c(K)
         waves = o.udiv(bm, wm) * o.udiv(bn, wn)
@@ -288,6 +295,11 @@ def _gemm_constraints(arch, M: int, N: int, K: int, type_size: int):
             o.implies(o.eq(direct, c(1)), o.uge(st, c(2))),
             o.implies(o.eq(direct, c(0)), o.ule(st, c(2))),
             o.ule(st, o.udiv(k_, bk)),
+            # the 16x16x32 body is written for the direct ring; its k-steps are 32 deep, and
+            # with one k-step per K-tile it takes two tiles per loop iteration
+            o.implies(o.eq(mfma, c(16)), o.eq(direct, c(1))),
+            o.implies(o.all_of(o.eq(mfma, c(16)), o.eq(bk, c(32))),
+                      o.eq(o.urem(o.udiv(k_, bk), c(2)), c(0))),
             # 1 to 16 waves per workgroup
             o.uge(threads, c(wave)), o.ule(threads, c(arch.max_threads_per_block)),
             # cooperative 16-byte loads (and epilogue stores) evenly cover the tiles
@@ -304,9 +316,10 @@ def _gemm_constraints(arch, M: int, N: int, K: int, type_size: int):
         # as in gemm_hip.est_regs_per_thread
         acc = o.udiv(wm * wn, c(wave))
         frags = 4 * (o.udiv(wm, c(32)) + o.udiv(wn, c(32)))
+        frags16 = 4 * (o.udiv(wm, c(16)) + 2 * o.udiv(wn, c(16)))  # A once, B twice
         chunks = o.udiv(o.udiv(bm * bk + bk * bn, c(8)), threads)
         staging = o.ite(o.eq(direct, c(1)), chunks, chunks * 4)
-        regs = acc + 2 * frags + staging + 40
+        regs = acc + o.ite(o.eq(mfma, c(16)), frags16, 2 * frags) + staging + 40
         regs8 = o.udiv(regs + 7, c(8)) * 8
         waves_per_simd = o.udiv(waves + (simds - 1), c(simds))
         out += [o.ule(regs, c(min(arch.vgprs_per_simd, SPILL_FREE_EST_REGS))),
@@ -322,7 +335,7 @@ def _gemm_constraints(arch, M: int, N: int, K: int, type_size: int):
     return build
 
 
-def solve_gemm_tc(arch, M: int, N: int, K: int, type_size: int = 2, count: int = 8192,
+def solve_gemm_tc(arch, M: int, N: int, K: int, type_size: int = 2, count: int = 65536,
                   backend: str = "auto"):
     """
     Enumerate FP16 MFMA GEMM tile configurations (see `GemmConfig`).
@@ -340,7 +353,7 @@ def solve_gemm_tc(arch, M: int, N: int, K: int, type_size: int = 2, count: int =
 
     tiles = _enumerate(GEMM_DOMAINS, _gemm_constraints(arch, M, N, K, type_size), count, backend)
     results = []
-    for bm, bn, bk, wm, wn, st, epi, direct in tiles:
+    for bm, bn, bk, wm, wn, st, epi, direct, mfma in tiles:
         # The rasterisation group only needs to divide the workgroup rows and the
         # XCD remap needs a multiple of 8 workgroups; neither interacts with the
         # other constraints, so both are expanded here (reference: Solver.py:550-558).
@@ -350,10 +363,14 @@ def solve_gemm_tc(arch, M: int, N: int, K: int, type_size: int = 2, count: int =
                 continue
             cfg = GemmConfig(BM=bm, BN=bn, BK=bk, warp_m=wm, warp_n=wn, stages=st,
                              raster=ras, epi_smem=bool(epi), xcd=xcd or ras == 0,
-                             direct=bool(direct))
+                             direct=bool(direct), mfma=mfma)
             # a grid that leaves a partial last wave may split its tiles in four; the
             # block order (raster 0) needs whole rounds of 8 sub-blocks of 8 x 4 tiles
-            for cand in (cfg, replace(cfg, tail=True, xcd=True)):
+            cands = [cfg, replace(cfg, tail=True, xcd=True)]
+            if mfma == 16 and wm >= 64:
+                # the barrier of a K-tile after half of the row blocks of its last k-step
+                cands += [replace(c, early=wm // 32) for c in cands]
+            for cand in cands:
                 if ras == 0 or cand.tail:
                     try:
                         check_config(cand, M, N, K)

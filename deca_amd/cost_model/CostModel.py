@@ -241,7 +241,7 @@ def rank_gemm_configs(configs, arch, M: int, N: int, K: int, top_n: int | None =
                       per_tile: int | None = None):
     """Sort FP16 MFMA GEMM configs by `gemm_tc_score` (best first).
 
-    `per_tile` keeps only that many tile orders (`raster`) of each tile set: the orders of
+    `per_tile` keeps only that many tile orders (`raster`, and barrier positions `early`) of each tile set: the orders of
     one tile set score within a percent or two of each other, so that a plain top-N would
     be spent on the six orders of the one or two best tile sets."""
     ranked = sorted(configs, key=lambda c: gemm_tc_score(c, arch, M, N, K), reverse=True)
@@ -250,7 +250,7 @@ def rank_gemm_configs(configs, arch, M: int, N: int, K: int, top_n: int | None =
 
         seen, kept = {}, []
         for c in ranked:
-            key = replace(c, raster=1)
+            key = replace(c, raster=1, early=0)
             seen[key] = seen.get(key, 0) + 1
             if seen[key] <= per_tile:
                 kept.append(c)

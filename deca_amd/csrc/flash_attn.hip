@@ -42,6 +42,11 @@
 // (DECA_LAZY_TAU), which leaves O / l the same quotient with p <= 2^tau
 // instead of p <= 1 and makes alpha exactly 1 for almost every tile.
 #include <hip/hip_runtime.h>
+
+// The direct-to-LDS loads below set M0 inside their asm statement and declare it
+// clobbered, so that the compiler never assumes an M0 value of its own survives one;
+// clang notes that M0 is a reserved register, which is the point.
+#pragma clang diagnostic ignored "-Winline-asm"
 #include <type_traits>
 #include <utility>
 
@@ -208,7 +213,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                  :
                  : "v"(voff), "s"(origin), "s"(lds_addr)
-                 : "memory");
+                 : "memory", "m0");
   };
   auto issue_k = [&](int j, int slot) __attribute__((always_inline)) {
     const _Float16* origin = k_base + static_cast<size_t>(j) * BC * D_;

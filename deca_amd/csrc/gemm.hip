@@ -33,6 +33,11 @@
 //   operand) so that each lane ends up with 4 consecutive n of one row of C.
 #include <hip/hip_runtime.h>
 
+// The direct-to-LDS loads below set M0 inside their asm statement and declare it
+// clobbered, so that the compiler never assumes an M0 value of its own survives one;
+// clang notes that M0 is a reserved register, which is the point.
+#pragma clang diagnostic ignored "-Winline-asm"
+
 #ifndef DECA_BM
 #error "gemm.hip is a template: define the DECA_* macros"
 #endif
@@ -54,17 +59,32 @@
 // 3:0 and 15:14, expcnt 6:4 and lgkmcnt 11:8 left at "no wait").
 #define DECA_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (((n) >> 4) << 14) | 0x0F70)
 
+#ifndef DECA_MFMA16
+#define DECA_MFMA16 0  // 1: v_mfma_f32_16x16x32 tiles instead of 32x32x16
+#endif
+#ifndef DECA_EARLY_GROUPS
+#define DECA_EARLY_GROUPS 0  // 16x16x32 body: MFMA groups of a K-tile's last k-step issued before its barrier
+#endif
 #if DECA_BF16
 typedef __bf16 elem_t;
+#if DECA_MFMA16
+#define DECA_MFMA __builtin_amdgcn_mfma_f32_16x16x32_bf16
+#else
 #define DECA_MFMA __builtin_amdgcn_mfma_f32_32x32x16_bf16
+#endif
 #else
 typedef _Float16 elem_t;
+#if DECA_MFMA16
+#define DECA_MFMA __builtin_amdgcn_mfma_f32_16x16x32_f16
+#else
 #define DECA_MFMA __builtin_amdgcn_mfma_f32_32x32x16_f16
+#endif
 #endif
 typedef elem_t half8 __attribute__((ext_vector_type(8)));
 typedef elem_t half4 __attribute__((ext_vector_type(4)));
 typedef short short4v __attribute__((ext_vector_type(4)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) short4v* lds_s4_ptr;
 typedef const __attribute__((address_space(1))) void* gptr;

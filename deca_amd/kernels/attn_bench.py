@@ -10,75 +10,106 @@ seeds a CUDA generator, attn_bench.py:73-78, whose stream is device specific).
 
 import math
 import time
-from typing import Callable
 
-# FlashAttention-2 paper setup: hidden = 2048, batch * seqlen = 16k.
+# Sweep grid of the FlashAttention-2 paper, as the reference uses it
+# (attn_bench.py:14-27): 16k tokens per batch at a hidden size of 2048, i.e.
+# head_dim x heads = 2048 and batch x seqlen = 16384.
+FA_TOKENS = 16384
+FA_HIDDEN = 2048
 FA_SEQLENS = [512, 1024, 2048, 4096, 8192, 16384]
-FA_HEADDIM_HEADS = [(64, 32), (128, 16)]
+FA_HEADDIM_HEADS = [(D, FA_HIDDEN // D) for D in (64, 128)]
 
 
 def standard_shapes():
-    """Returns a list of (B, H, S, D)."""
-    shapes = []
-    for D, H in FA_HEADDIM_HEADS:
-        for S in FA_SEQLENS:
-            shapes.append((16384 // S, H, S, D))
-    return shapes
+    """The sweep grid as (B, H, S, D) tuples, head dims outermost."""
+    return [(FA_TOKENS // S, H, S, D) for D, H in FA_HEADDIM_HEADS for S in FA_SEQLENS]
 
 
 def attn_flops(B: int, H: int, S_q: int, S_kv: int, D: int, causal: bool = False) -> float:
-    flops = 4.0 * B * H * S_q * S_kv * D
-    return flops / 2 if causal else flops
+    """Two S_q x S_kv x D products per head, 2 FLOPs per multiply-add; a causal
+    mask leaves half of the score matrix (reference: attn_bench.py:30-32)."""
+    products = 2.0 * (B * H) * S_q * S_kv * D
+    return products if causal else 2.0 * products
 
 
-def bench_cuda(
-    fn: Callable[[], None],
-    warmup_s: float = 0.3,
-    measure_s: float = 0.3,
-    min_iters: int = 20,
-) -> float:
-    """Median time of `fn` in seconds, measured with one event pair per call
-    on torch's current stream (which is the stream the kernels launch on).
+class _EventTimer:
+    """Times single calls on torch's current stream (the stream every kernel of
+    this package is launched on) with a reusable pool of event pairs."""
 
-    Warm-up and measurement are time based, as in the reference
-    (attn_bench.py:35-70): short warm-ups leave the GPU at a lower clock.
+    def __init__(self, pairs: int = 64):
+        import torch
+
+        self._torch = torch
+        self._pool = [self._pair() for _ in range(pairs)]
+
+    def _pair(self):
+        ev = self._torch.cuda.Event
+        return ev(enable_timing=True), ev(enable_timing=True)
+
+    def one(self, fn, slot: int = 0) -> float:
+        """Seconds of one call that starts on an idle stream."""
+        while slot >= len(self._pool):
+            self._pool.append(self._pair())
+        first, last = self._pool[slot]
+        first.record()
+        fn()
+        last.record()
+        last.synchronize()
+        return first.elapsed_time(last) * 1e-3
+
+    def spin(self, fn, seconds: float) -> float:
+        """Keeps calling `fn` for `seconds` of wall-clock time so that the clocks
+        settle; returns the duration of the last call."""
+        deadline = time.perf_counter() + seconds
+        last = self.one(fn)
+        while time.perf_counter() < deadline:
+            last = self.one(fn)
+        return last
+
+    def samples(self, fn, count: int) -> list:
+        return [self.one(fn, i % len(self._pool)) for i in range(count)]
+
+
+_timer = None
+
+
+def _event_timer() -> _EventTimer:
+    global _timer
+    if _timer is None:
+        _timer = _EventTimer()
+    return _timer
+
+
+def _median(values) -> float:
+    ordered = sorted(values)
+    return ordered[len(ordered) // 2]
+
+
+def bench_cuda(fn, warmup_s: float = 0.3, measure_s: float = 0.3, min_iters: int = 20) -> float:
+    """Median seconds per call of `fn`.
+
+    Same measurement as the reference's helper of this name
+    (attn_bench.py:35-70): a warm-up that lasts `warmup_s` of wall-clock time
+    (a fixed number of calls leaves the GPU at a low clock for short kernels),
+    then about `measure_s` worth of calls and never fewer than `min_iters`, each
+    bracketed by its own event pair and followed by a synchronisation; the
+    result is the median of those single-call times.
     """
-    import torch
-
-    fn()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    while time.perf_counter() - t0 < warmup_s:
-        fn()
-        torch.cuda.synchronize()
-    probe_start = torch.cuda.Event(enable_timing=True)
-    probe_end = torch.cuda.Event(enable_timing=True)
-    probe_start.record()
-    fn()
-    probe_end.record()
-    probe_end.synchronize()
-    per_call = max(probe_start.elapsed_time(probe_end) / 1e3, 1e-6)
-    iters = max(min_iters, int(measure_s / per_call))
-    times = []
-    for _ in range(iters):
-        start = torch.cuda.Event(enable_timing=True)
-        end = torch.cuda.Event(enable_timing=True)
-        start.record()
-        fn()
-        end.record()
-        end.synchronize()
-        times.append(start.elapsed_time(end) / 1e3)
-    times.sort()
-    return times[len(times) // 2]
+    timer = _event_timer()
+    settled = max(timer.spin(fn, warmup_s), 1e-6)
+    count = max(int(min_iters), int(measure_s / settled))
+    return _median(timer.samples(fn, count))
 
 
 def bench_interleaved(fns: dict, rounds: int = 3) -> dict:
-    """Times several callables alternately; returns the median per name (seconds)."""
-    samples = {name: [] for name in fns}
+    """Median of `rounds` bench_cuda results per entry of `fns`, the entries
+    taking turns in every round so that drift (clocks, temperature) hits all of
+    them alike (reference: attn_bench.py:94-100)."""
+    per_name = {name: [] for name in fns}
     for _ in range(rounds):
-        for name, fn in fns.items():
-            samples[name].append(bench_cuda(fn))
-    return {name: sorted(ts)[len(ts) // 2] for name, ts in samples.items()}
+        for name in per_name:
+            per_name[name].append(bench_cuda(fns[name]))
+    return {name: _median(seen) for name, seen in per_name.items()}
 
 
 def make_qkv(B: int, H: int, S_q: int, S_kv: int, D: int, dtype=None, seed: int = 0,
@@ -102,11 +133,27 @@ def make_qkv_cpu(B: int, H: int, S_q: int, S_kv: int, D: int, dtype=None, seed: 
     return make_qkv(B, H, S_q, S_kv, D, dtype, seed, "cpu")
 
 
+# Which torch attention back end `sdpa_flash` ran last ("flash" when the pin below
+# held, "default" when torch chose); drivers print it beside the ratio column.
+SDPA_BACKEND = "flash"
+
+
 def sdpa_flash(q, k, v, causal: bool = False, scale: float | None = None):
-    """torch's fused attention on the device (the baseline the tuner reports
-    against; reference: attn_bench.py:81-83)."""
+    """torch's fused attention restricted to its flash back end, the baseline the
+    tuner reports against (reference: attn_bench.py:81-83).  Where this torch
+    build has no flash kernel for the inputs, torch picks the back end and
+    `SDPA_BACKEND` says so."""
+    global SDPA_BACKEND
     import torch.nn.functional as F
 
+    if SDPA_BACKEND == "flash":
+        try:
+            from torch.nn.attention import SDPBackend, sdpa_kernel
+
+            with sdpa_kernel(SDPBackend.FLASH_ATTENTION):
+                return F.scaled_dot_product_attention(q, k, v, is_causal=causal, scale=scale)
+        except (ImportError, RuntimeError):
+            SDPA_BACKEND = "default"
     return F.scaled_dot_product_attention(q, k, v, is_causal=causal, scale=scale)
 
 

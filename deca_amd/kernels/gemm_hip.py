@@ -55,6 +55,13 @@ class GemmConfig:
     # (BM/2 x BN/2, wave tiles halved), so that they fill the whole GPU for a quarter of
     # a tile's time instead of a quarter of the GPU for a whole one
     tail: bool = False
+    # MFMA tile: 32 -> v_mfma_f32_32x32x16, 16 -> v_mfma_f32_16x16x32 (less energy per
+    # FLOP on this board; needs BK = 64 and the direct-to-LDS ring)
+    mfma: int = 32
+    # 16x16x32 body: row-block groups of a K-tile's last k-step that issue before the
+    # barrier which publishes the next tile (a later barrier gives the loads more time,
+    # and leaves fewer MFMAs to cover the first fragment reads of the next tile)
+    early: int = 0
 
     @property
     def num_warps(self) -> int:
@@ -74,6 +81,8 @@ class GemmConfig:
             + ("" if self.xcd else ",xcd=0")
             + ("" if self.direct else ",direct=0")
             + (",tail=1" if self.tail else "")
+            + (f",mfma={self.mfma}" if self.mfma != 32 else "")
+            + (f",early={self.early}" if self.early else "")
         )
 
 
@@ -101,10 +110,13 @@ def est_regs_per_thread(cfg: GemmConfig) -> int:
     one set of A / B fragments (4 VGPRs per 32-row tile), the global->LDS
     staging registers and addressing."""
     acc = cfg.warp_m * cfg.warp_n // WAVE
-    frags = 4 * (cfg.warp_m // MFMA_M + cfg.warp_n // MFMA_M)  # one of the two sets
     chunks = (cfg.BM * cfg.BK + cfg.BK * cfg.BN) // 8 // cfg.threads
     # direct loads keep one offset register per chunk, staged loads four data registers
     staging = chunks if cfg.direct else chunks * 4
+    if cfg.mfma == 16:
+        # one set of A fragments (refilled in place), two of B, 4 VGPRs per 16-row tile
+        return acc + 4 * (cfg.warp_m // 16 + 2 * (cfg.warp_n // 16)) + staging + 40
+    frags = 4 * (cfg.warp_m // MFMA_M + cfg.warp_n // MFMA_M)  # one of the two sets
     return acc + 2 * frags + staging + 40
 
 
@@ -142,10 +154,18 @@ def target_waves_per_simd(cfg: GemmConfig) -> int:
 
 
 def check_config(cfg: GemmConfig, M: int, N: int, K: int, max_smem: int = MAX_LDS) -> None:
-    assert cfg.stages in ((2, 3, 4) if cfg.direct else (1, 2))
+    assert cfg.stages in ((2, 3, 4, 5) if cfg.direct else (1, 2))
     assert K // cfg.BK >= cfg.stages
     assert smem_bytes(cfg) <= max_smem
     assert cfg.BK in (32, 64)
+    assert cfg.mfma in (32, 16)
+    if cfg.mfma == 16:
+        # k-steps of 32; with one k-step per K-tile the main loop takes two tiles at a time
+        assert cfg.direct
+        assert cfg.BK == 64 or (K // cfg.BK) % 2 == 0
+        assert 0 <= cfg.early < cfg.warp_m // 16
+    else:
+        assert cfg.early == 0
     assert cfg.warp_m % MFMA_M == 0 and cfg.warp_n % MFMA_M == 0
     assert cfg.BM % cfg.warp_m == 0 and cfg.BN % cfg.warp_n == 0
     assert cfg.BN >= 64
@@ -203,6 +223,9 @@ def make_gemm_tc(M: int, N: int, K: int, cfg: GemmConfig, dtype: str = "float16"
         "DECA_DIRECT": int(cfg.direct), "DECA_BF16": int(dtype == "bfloat16"),
         "DECA_MIN_WAVES": target_waves_per_simd(cfg),
     }
+    if cfg.mfma == 16:
+        defines["DECA_MFMA16"] = 1
+        defines["DECA_EARLY_GROUPS"] = cfg.early
     workgroups = (M // cfg.BM) * (N // cfg.BN)
     if cfg.tail:
         r = tail_tiles(cfg, M, N)

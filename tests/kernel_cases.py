@@ -84,6 +84,21 @@ GEMM_CASES = [
     # tail: the 64 tiles of the partial last wave (576 = 512 + 64) as 256 quarter tiles
     (3072, 3072, 256, GemmConfig(128, 128, 64, 64, 64, 2, 4, True, True, True, True)),
     (3072, 3072, 256, GemmConfig(128, 128, 64, 64, 64, 2, 1, False, True, True, True)),
+    # 16x16x32 MFMA body: ring depths 2..5, one or two k-steps per K-tile, both wave
+    # orientations, the barrier before or inside the last k-step, both epilogues, the block
+    # order and the tail split
+    (512, 512, 512, GemmConfig(256, 256, 64, 128, 64, 2, 1, True, False, True, mfma=16)),
+    (512, 512, 512, GemmConfig(256, 256, 64, 64, 128, 2, 2, False, False, True, mfma=16, early=2)),
+    (512, 1024, 256, GemmConfig(256, 256, 32, 128, 64, 3, 2, True, True, True, mfma=16, early=4)),
+    (512, 512, 512, GemmConfig(256, 256, 32, 128, 64, 4, 1, False, False, True, mfma=16)),
+    (512, 512, 512, GemmConfig(256, 256, 32, 64, 128, 5, 1, True, False, True, mfma=16, early=3)),
+    (512, 512, 512, GemmConfig(128, 128, 64, 64, 64, 3, 4, False, True, True, mfma=16, early=1)),
+    (384, 640, 1088, GemmConfig(128, 128, 64, 64, 32, 4, 1, True, False, True, mfma=16)),
+    (256, 256, 128, GemmConfig(64, 64, 64, 32, 32, 2, 1, False, False, True, mfma=16)),
+    (128, 192, 64, GemmConfig(64, 64, 32, 32, 64, 2, 2, False, False, True, mfma=16)),
+    (3072, 4096, 128, GemmConfig(128, 128, 64, 64, 64, 2, 0, False, True, True, mfma=16, early=2)),
+    (3072, 3072, 256, GemmConfig(128, 128, 64, 64, 64, 2, 0, True, True, True, True, mfma=16)),
+    (3072, 3072, 256, GemmConfig(128, 128, 64, 64, 64, 2, 4, True, True, True, True, mfma=16, early=2)),
     # VGPR-staged ring
     (3840, 3840, 128, GemmConfig(128, 128, 64, 64, 64, 1, 2, True, True, False, True)),  # tail
     (512, 512, 512, GemmConfig(256, 256, 64, 128, 128, 2, 1, False, False, False)),
@@ -99,6 +114,7 @@ GEMM_FULL = [
     (8192, 8192, 8192, GemmConfig(256, 256, 32, 128, 128, 3, 8, False, True, True)),
     (8192, 8192, 8192, GemmConfig(256, 256, 64, 128, 64, 2, 0, True, True, True)),
     (6144, 6144, 6144, GemmConfig(256, 256, 64, 128, 64, 2, 8, True, True, True, True)),
+    (8192, 8192, 8192, GemmConfig(256, 256, 64, 128, 64, 2, 0, True, True, True, mfma=16, early=4)),
 ]
 
 
@@ -108,6 +124,8 @@ GEMM_BF16_CASES = [
     (512, 1024, 256, GemmConfig(128, 128, 32, 64, 64, 3, 2, True, True, True)),
     (256, 256, 192, GemmConfig(64, 64, 64, 32, 32, 1, 1, False, False, False)),
     (3072, 3072, 256, GemmConfig(128, 128, 64, 64, 64, 2, 0, True, True, True, True)),  # block order + tail
+    (512, 512, 512, GemmConfig(256, 256, 64, 128, 64, 2, 1, True, False, True, mfma=16, early=4)),
+    (512, 1024, 256, GemmConfig(128, 128, 32, 64, 64, 3, 2, False, True, True, mfma=16)),
 ]
 
 

@@ -126,11 +126,11 @@ def test_gemm_ranking_can_limit_the_tile_orders_per_tile_set():
     cfgs = Solver.solve_gemm_tc(ARCH, n, n, n)
     plain = cm.rank_gemm_configs(cfgs, ARCH, n, n, n, top_n=12)
     spread = cm.rank_gemm_configs(cfgs, ARCH, n, n, n, top_n=12, per_tile=3)
-    tiles = lambda cs: {replace(c, raster=1) for c in cs}  # noqa: E731
+    tiles = lambda cs: {replace(c, raster=1, early=0) for c in cs}  # noqa: E731
     assert len(tiles(spread)) >= 4 > len(tiles(plain)) - 1
     assert spread[0] == plain[0]
     for t in tiles(spread):
-        assert sum(replace(c, raster=1) == t for c in spread) <= 3
+        assert sum(replace(c, raster=1, early=0) == t for c in spread) <= 3
     # the order of what is kept is still the score order
     scores = [cm.gemm_tc_score(c, ARCH, n, n, n) for c in spread]
     assert scores == sorted(scores, reverse=True)

@@ -89,13 +89,13 @@ def test_gemm_configs_are_valid(n):
         assert gm.GemmConfig(256, 256, 64, 128, 64, 2, 4, False, True, True) in configs
     # independent enumeration of the tile sets
     tiles = set()
-    for bm, bn, bk, wm, wn, st, epi, direct in itertools.product(
-            (64, 128, 256), (64, 128, 256), (32, 64), (32, 64, 128), (32, 64, 128), (1, 2, 3, 4),
-            (False, True), (False, True)):
+    for bm, bn, bk, wm, wn, st, epi, direct, mfma in itertools.product(
+            (64, 128, 256), (64, 128, 256), (32, 64), (32, 64, 128), (32, 64, 128), (1, 2, 3, 4, 5),
+            (False, True), (False, True), (32, 16)):
         if bm % wm or bn % wn:
             continue
         xcd = ((n // bm) * (n // bn)) % 8 == 0
-        cfg = gm.GemmConfig(bm, bn, bk, wm, wn, st, 1, epi, xcd, direct)
+        cfg = gm.GemmConfig(bm, bn, bk, wm, wn, st, 1, epi, xcd, direct, mfma=mfma)
         try:
             gm.check_config(cfg, n, n, n)
         except AssertionError:
@@ -105,9 +105,13 @@ def test_gemm_configs_are_valid(n):
         regs = (gm.est_regs_per_thread(cfg) + 7) // 8 * 8
         if regs * -(-cfg.num_warps // 4) > 512 or gm.est_regs_per_thread(cfg) > gm.SPILL_FREE_EST_REGS:
             continue
-        tiles.add((bm, bn, bk, wm, wn, st, epi, direct))
-    got = {(c.BM, c.BN, c.BK, c.warp_m, c.warp_n, c.stages, c.epi_smem, c.direct) for c in configs}
+        tiles.add((bm, bn, bk, wm, wn, st, epi, direct, mfma))
+    got = {(c.BM, c.BN, c.BK, c.warp_m, c.warp_n, c.stages, c.epi_smem, c.direct, c.mfma)
+           for c in configs}
     assert got == tiles
+    # the 16x16x32 body offers its barrier before or in the middle of a tile's last k-step
+    assert {c.early for c in configs if c.mfma == 16 and c.warp_m == 128} == {0, 4}
+    assert all(c.early == 0 for c in configs if c.mfma == 32)
     # every rasterisation that divides the grid is offered for every tile set
     for c in configs:
         if c.tail:
@@ -117,8 +121,8 @@ def test_gemm_configs_are_valid(n):
         if gm_ % 8 == 0 and gn_ % 4 == 0 and (gm_ * gn_) % 256 == 0:
             want.add(0)
         have = {d.raster for d in configs if not d.tail and
-                (d.BM, d.BN, d.BK, d.warp_m, d.warp_n, d.stages, d.epi_smem, d.direct)
-                == (c.BM, c.BN, c.BK, c.warp_m, c.warp_n, c.stages, c.epi_smem, c.direct)}
+                (d.BM, d.BN, d.BK, d.warp_m, d.warp_n, d.stages, d.epi_smem, d.direct, d.mfma, d.early)
+                == (c.BM, c.BN, c.BK, c.warp_m, c.warp_n, c.stages, c.epi_smem, c.direct, c.mfma, c.early)}
         assert have == want
         break
 
@@ -247,7 +251,7 @@ def test_gemm_tail_split_is_offered_where_a_partial_wave_remains():
     quarter tiles.  A grid that fills its waves exactly gets no such variant."""
     cfgs = Solver.solve_gemm_tc(ARCH, 6144, 6144, 6144)
     split = [c for c in cfgs if c.tail]
-    assert split and all(str(c).endswith(",tail=1") for c in split)
+    assert split and all(",tail=1" in str(c) for c in split)
     big = gm.GemmConfig(256, 256, 64, 128, 64, 2, 8, True, True, True, tail=True)
     assert big in split and gm.tail_tiles(big, 6144, 6144) == 64
     spec = gm.make_gemm_tc(6144, 6144, 6144, big)
