@@ -235,15 +235,48 @@ def run_fa(wl, steps, warmup, with_cpu):
     return res
 
 
-def _measured_traffic(name):
+def _measured_traffic(name, config):
     """HBM-side bytes per launch measured with rocprofv3 counters (see
-    deca_amd/measured_traffic.json and profiles/), or None when not recorded."""
+    deca_amd/measured_traffic.json and profiles/).  The figure belongs to the
+    kernel configuration it was measured on: None when nothing is recorded for
+    the workload or the record is for another configuration than the timed one."""
     path = os.path.join(ROOT, "deca_amd", "measured_traffic.json")
     if not os.path.exists(path):
         return None
     with open(path) as f:
         entry = json.load(f).get("workloads", {}).get(name)
-    return entry["traffic_bytes"] if entry else None
+    if not entry or entry.get("config") != config:
+        return None
+    return entry["traffic_bytes"]
+
+
+# The roofline fractions the task sets for the gated workloads (of 8 TB/s HBM
+# bandwidth, or of 2.5 PFLOP/s dense fp16 MFMA).
+TARGET_FRAC = {
+    "rmsnorm_bf16_16384x4096": 0.80,
+    "softmax_fp16_16384x4096": 0.80,
+    "rmsnorm_fp16_8192x8192": 0.80,
+    "gemm_fp16_8192": 0.70,
+    "fa_fp16_b4h16s4096d128": 0.55,
+}
+
+
+def _compact(res):
+    """What a reader needs to recompute one workload's roofline fraction."""
+    rf = res["roofline"]
+    row = {
+        "value": round(res["value"], 2), "unit": res["unit"],
+        "ms_per_step": round(res["ms_per_step"], 5),
+        "kernel_us": round(rf["kernel_us"], 3),
+        "work": rf.get("algorithmic_bytes", rf.get("algorithmic_flops")),
+        "achieved": round(rf["achieved"], 2), "peak": rf["peak"], "frac": round(rf["frac"], 4),
+        "traffic": rf["traffic"], "kernel_config": res["config"],
+    }
+    target = TARGET_FRAC.get(res["workload"])
+    if target is not None:
+        row["target_frac"] = target
+        row["target_met"] = bool(rf["frac"] >= target)
+    return row
 
 
 def run(wl, steps, warmup, with_cpu=True):
@@ -251,7 +284,7 @@ def run(wl, steps, warmup, with_cpu=True):
     print(f"[bench] {wl['name']} ...", file=sys.stderr, flush=True)
     res = {"rowwise": run_rowwise, "gemm": run_gemm, "fa": run_fa}[wl["kind"]](
         wl, steps, warmup, with_cpu)
-    res["roofline"]["traffic"] = _measured_traffic(wl["name"])
+    res["roofline"]["traffic"] = _measured_traffic(wl["name"], res["config"])
     print(f"[bench] {wl['name']}: {res['value']:.1f} {res['unit']} "
           f"({100 * res['roofline']['frac']:.1f}% of peak) in {time.perf_counter() - t0:.1f} s",
           file=sys.stderr, flush=True)
@@ -296,15 +329,35 @@ def main():
     }
     if "cpu_baseline" in head:
         out["cpu_baseline"] = head["cpu_baseline"]
+    results = [head]
     if not args.no_extra:
         # the other benchmark configurations, with fewer steps each so that the
         # default run stays within a few minutes
         k = max(5, min(args.steps, 30))
-        out["results"] = [head] + [
-            run(wl, k, min(args.warmup, 5), not args.no_cpu)
-            for name, wl in wls.items() if name != args.workload
-        ]
-    print(json.dumps(out))
+        results += [run(wl, k, min(args.warmup, 5), not args.no_cpu)
+                    for name, wl in wls.items() if name != args.workload]
+        out["results"] = results
+    # Every workload of the run in compact form inside the two objects a reader of
+    # the record is sure to keep, and which of the stated targets were met.
+    out["roofline"] = dict(head["roofline"], all={r["workload"]: _compact(r) for r in results})
+    if "cpu_baseline" in head:
+        out["cpu_baseline"] = dict(
+            head["cpu_baseline"],
+            all={r["workload"]: r["cpu_baseline"] for r in results if "cpu_baseline" in r})
+    gated = {r["workload"]: _compact(r) for r in results if r["workload"] in TARGET_FRAC}
+    out["config"]["targets_met"] = sorted(n for n, c in gated.items() if c["target_met"])
+    out["config"]["targets_missed"] = {n: {"frac": c["frac"], "target": c["target_frac"]}
+                                       for n, c in gated.items() if not c["target_met"]}
+    print(json.dumps(out), flush=True)
+    # one line per workload, last on stderr
+    print(f"[bench] {'workload':32s} {'value':>10s} {'unit':8s} {'kernel us':>10s} {'frac':>6s} "
+          f"{'target':>6s}  config", file=sys.stderr)
+    for r in results:
+        c = _compact(r)
+        tgt = f"{c['target_frac']:.2f}" if "target_frac" in c else "  -"
+        print(f"[bench] {r['workload']:32s} {c['value']:10.1f} {c['unit']:8s} {c['kernel_us']:10.2f} "
+              f"{c['frac']:6.3f} {tgt:>6s}  {c['kernel_config']}", file=sys.stderr)
+    sys.stderr.flush()
 
 
 if __name__ == "__main__":

@@ -1,0 +1,173 @@
+"""
+Measures what one MI355X sustains on nothing but roofline-limited work: the
+ceilings behind the constants of `arch/MI355X.py` and behind every "fraction of
+peak" this package reports.  The reference pastes such measurements into its
+arch files as comments (arch/H20.py:35-60); here they can be taken again:
+
+    python -m deca_amd.arch.ceilings             # HBM streams and matrix-pipe loops
+    python -m deca_amd.arch.ceilings --sclk      # + shader clock while the tuned 8192^3 GEMM runs
+
+- HBM: a 16-byte-per-lane copy, a read-only and a write-only stream of 128 MiB
+  buffers, rotating over 8 buffer pairs (2 GiB, several times the 256 MiB Infinity
+  Cache) so that every launch streams from memory.
+- Matrix pipe: register-only loops of v_mfma_f32_32x32x16_f16 and
+  v_mfma_f32_16x16x32_f16 (no memory traffic) on N(0,1) and on all-zero operands:
+  with real data the board's power limit, not its 2.4 GHz clock, sets the rate.
+"""
+
+from __future__ import annotations
+
+import argparse
+import itertools
+import subprocess
+import sys
+import threading
+import time
+
+from deca_amd.kernels.build import cached_build, make_spec
+
+TEMPLATE = "ceilings.hip"
+STREAM_BYTES = 128 * 1024 * 1024
+ROTATE = 8
+MFMA_ITERS = 4096
+MFMA_FLOPS = {3: 2 * 32 * 32 * 16, 4: 2 * 16 * 16 * 32}
+
+
+def stream_spec(mode: int, threads: int, unroll: int, nt: int, wgs: int):
+    chunks = STREAM_BYTES // 16
+    grid = wgs if wgs else -(-chunks // (threads * unroll))
+    return make_spec(TEMPLATE, {"DECA_CEILING": mode, "DECA_THREADS": threads, "DECA_CHUNKS": chunks,
+                                "DECA_UNROLL": unroll, "DECA_NT": nt},
+                     (grid, 1, 1), (threads, 1, 1), 2, options=[])
+
+
+def mfma_spec(mode: int, nacc: int, blocks: int):
+    return make_spec(TEMPLATE, {"DECA_CEILING": mode, "DECA_THREADS": 256, "DECA_ITERS": MFMA_ITERS,
+                                "DECA_NACC": nacc}, (blocks, 1, 1), (256, 1, 1), 2, options=[])
+
+
+STREAM_VARIANTS = [(t, u, nt, w) for t, u, nt, w in itertools.product(
+    (256, 512, 1024), (1, 2, 4), (0, 1), (0, 2048))]
+MFMA_VARIANTS = [(3, 8, 1024), (3, 8, 2048), (4, 16, 1024), (4, 16, 2048)]
+
+
+def all_specs():
+    specs = [stream_spec(m, *v) for m in (0, 1, 2) for v in STREAM_VARIANTS]
+    return specs + [mfma_spec(*v) for v in MFMA_VARIANTS]
+
+
+def build():
+    from concurrent.futures import ThreadPoolExecutor
+
+    unique = {spec.key(): spec for spec in all_specs()}  # grids differ, code objects do not
+    with ThreadPoolExecutor(8) as pool:
+        list(pool.map(cached_build, unique.values()))
+
+
+def measure_streams(out=sys.stdout):
+    import torch
+
+    from deca_amd.driver.driver import load_kernel
+
+    n = STREAM_BYTES // 4
+    bufs = [(torch.randn(n, device="cuda"), torch.empty(n, device="cuda")) for _ in range(ROTATE)]
+    names = {0: "copy", 1: "read only", 2: "write only"}
+    moved = {0: 2 * STREAM_BYTES, 1: STREAM_BYTES, 2: STREAM_BYTES}
+    for mode in (0, 1, 2):
+        best = (0.0, None)
+        for v in STREAM_VARIANTS:
+            spec = stream_spec(mode, *v)
+            kern = load_kernel(spec, cached_build(spec))
+            kern.time(bufs, ROTATE)
+            t = min(kern.time(bufs, 4 * ROTATE) for _ in range(3))
+            rate = moved[mode] / t / 1e9
+            if rate > best[0]:
+                best = (rate, v, t)
+        rate, (threads, unroll, nt, wgs), t = best
+        print(f"HBM {names[mode]:10s}: {rate:7.0f} GB/s ({t * 1e6:.1f} us per {STREAM_BYTES >> 20} MiB"
+              f"{' in + out' if mode == 0 else ''}; best of {len(STREAM_VARIANTS)} variants: "
+              f"{threads} lanes, {unroll} in flight, {'non-temporal' if nt else 'plain'}, "
+              f"{'grid-stride over ' + str(wgs) + ' workgroups' if wgs else 'one pass per lane'})",
+              file=out, flush=True)
+
+
+def measure_mfma(out=sys.stdout):
+    import torch
+
+    from deca_amd.driver.driver import load_kernel
+
+    operands = {"N(0,1)": torch.randn(4096 * 8, device="cuda").half(),
+                "zeros": torch.zeros(4096 * 8, device="cuda").half()}
+    for mode, nacc, blocks in MFMA_VARIANTS:
+        spec = mfma_spec(mode, nacc, blocks)
+        kern = load_kernel(spec, cached_build(spec))
+        res = torch.empty(blocks * 256, device="cuda")
+        flops = blocks * 4 * MFMA_ITERS * nacc * MFMA_FLOPS[mode]
+        form = "32x32x16" if mode == 3 else "16x16x32"
+        for name, x in operands.items():
+            kern.time([(x, res)], 2)
+            t = min(kern.time([(x, res)], 5) for _ in range(3))
+            print(f"MFMA {form} f16, {blocks} workgroups x 4 waves x {nacc} tiles, {name:6s}: "
+                  f"{flops / t / 1e12:6.0f} TFLOP/s ({t * 1e3:.3f} ms)", file=out, flush=True)
+
+
+def _sclk():
+    try:
+        text = subprocess.run(["rocm-smi", "--showclocks"], capture_output=True, text=True,
+                              timeout=20).stdout
+    except (OSError, subprocess.SubprocessError) as err:
+        return f"rocm-smi failed: {err}"
+    return " | ".join(line.strip() for line in text.splitlines() if "sclk" in line)
+
+
+def measure_sclk(out=sys.stdout):
+    """Shader clock reported by rocm-smi while the tuned 8192^3 GEMM loops."""
+    import torch
+
+    from deca_amd import tuned
+    from deca_amd.kernels.gemm_hip import build_gemm_tc, make_gemm_tc
+
+    n = 8192
+    cfg = tuned.lookup(tuned.make_key("GEMM", (n, n, n), "float16", "gfx950", False))
+    kern = build_gemm_tc(make_gemm_tc(n, n, n, cfg))
+    print(f"idle: {_sclk()}", file=out, flush=True)
+    makers = {"U(-1,1)": lambda: (2 * torch.rand(n, n, device="cuda") - 1).half(),
+              "zeros": lambda: torch.zeros(n, n, device="cuda", dtype=torch.float16)}
+    for name, make in makers.items():
+        a, b = make(), make()
+        c = torch.empty(n, n, device="cuda", dtype=torch.float16)
+        stop = threading.Event()
+
+        def work():
+            while not stop.is_set():
+                for _ in range(50):
+                    kern(a, b, c)
+                torch.cuda.synchronize()
+
+        worker = threading.Thread(target=work)
+        worker.start()
+        for _ in range(3):
+            time.sleep(1.0)
+            print(f"GEMM {n}^3 [{cfg}] on {name}: {_sclk()}", file=out, flush=True)
+        stop.set()
+        worker.join()
+        t = kern.time([(a, b, c)], 20)
+        print(f"  -> {2 * n**3 / t / 1e12:.0f} TFLOP/s", file=out, flush=True)
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--build", action="store_true", help="compile the probe kernels and exit")
+    ap.add_argument("--sclk", action="store_true", help="also sample the shader clock under the GEMM")
+    args = ap.parse_args(argv)
+    build()
+    if args.build:
+        return
+    measure_streams()
+    measure_mfma()
+    if args.sclk:
+        measure_sclk()
+
+
+if __name__ == "__main__":
+    main()

@@ -25,7 +25,8 @@
 //                 second operand Q (32 queries x 16 d, kept in VGPRs);
 //                 a lane then holds ONE query column (lane % 32) and 16 key
 //                 rows per 32-key block, so the row max / row sum of the online
-//                 softmax are in-lane reductions plus one exchange with lane^32;
+//                 softmax are in-lane reductions plus one exchange with lane^32
+//                 (v_permlane32_swap);
 //   O^T = V^T P^T first operand V^T (32 d x 16 keys, transposing
 //                 ds_read_b64_tr_b16 of the row-major V tile), second operand
 //                 P^T taken straight from the S^T accumulator registers (its
@@ -136,6 +137,29 @@ __device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int
 template <int N, class F>
 __device__ __forceinline__ void static_for(F&& f) {
   static_for_impl(f, std::make_integer_sequence<int, (N > 0 ? N : 0)>{});
+}
+
+// The values of lanes l and l ^ 32 (the two 32-lane halves of the wave hold the two
+// halves of a query's keys): v_permlane32_swap on two copies of x leaves the lower
+// half's value in every lane of one copy and the upper half's in the other.  A vector
+// ALU instruction; the generic cross-lane shuffle would go through the LDS pipe.
+__device__ __forceinline__ void both_halves(float x, float& lower, float& upper) {
+  typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+  const unsigned u = __builtin_bit_cast(unsigned, x);
+  const u32x2 r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  const unsigned lo = r.x, hi = r.y;
+  lower = __builtin_bit_cast(float, lo);
+  upper = __builtin_bit_cast(float, hi);
+}
+__device__ __forceinline__ float max_halves(float x) {
+  float a, b;
+  both_halves(x, a, b);
+  return fmaxf(a, b);
+}
+__device__ __forceinline__ float sum_halves(float x) {
+  float a, b;
+  both_halves(x, a, b);
+  return a + b;
 }
 
 #define DECA_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (((n) >> 4) << 14) | 0x0F70)
@@ -341,7 +365,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
       for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
         for (int e = 0; e < 16; ++e) mx = fmaxf(mx, s_acc[kt][mq][e]);
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      mx = max_halves(mx);
       const float m_new = lazy_max(m_i[mq], mx);
       alpha[mq] = __builtin_amdgcn_exp2f((m_i[mq] - m_new) * SL2);
       m_i[mq] = m_new;
@@ -457,7 +481,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
       for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
         for (int e = 0; e < 16; ++e) mx = fmaxf(mx, s_acc[kt][mq][e]);
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      mx = max_halves(mx);
       const float m_new = lazy_max(m_i[mq], mx);
       alpha[mq] = __builtin_amdgcn_exp2f((m_i[mq] - m_new) * SL2);
       m_i[mq] = m_new;
@@ -593,7 +617,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
   auto finish_stats = [&](float (&mx)[MQ]) __attribute__((always_inline)) {
 #pragma unroll
     for (int mq = 0; mq < MQ; ++mq) {
-      const float mxx = fmaxf(mx[mq], __shfl_xor(mx[mq], 32, 64));
+      const float mxx = max_halves(mx[mq]);
       const float m_new = lazy_max(m_i[mq], mxx);
       alpha[mq] = __builtin_amdgcn_exp2f((m_i[mq] - m_new) * SL2);
       m_i[mq] = m_new;
@@ -867,7 +891,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
   _Float16* o_lds = reinterpret_cast<_Float16*>(lds) + wave * WQ * EPI_LD;
 #pragma unroll
   for (int mq = 0; mq < MQ; ++mq) {
-    const float l = l_i[mq] + __shfl_xor(l_i[mq], 32, 64);
+    const float l = sum_halves(l_i[mq]);
     const float inv = 1.0f / l;
     _Float16* o_row = EPI_LDS ? o_lds + (mq * 32 + l32) * EPI_LD + half * 4
                               : o_base + (mq * 32 + l32) * D_ + half * 4;

@@ -87,12 +87,23 @@ __device__ __forceinline__ float wave_allreduce(float v, Op op) {
   if (LANES >= 4) v = op(v, dpp_f<0x4E>(v));   // quad_perm [2,3,0,1]
   if (LANES >= 8) v = op(v, dpp_f<0x141>(v));  // row_half_mirror
   if (LANES >= 16) v = op(v, dpp_f<0x140>(v)); // row_mirror
+  // The last two steps pair 16-lane rows, then the 32-lane halves, with the row
+  // swaps of gfx950 (v_permlane16_swap / v_permlane32_swap on two copies of v:
+  // one copy ends up with the even rows' values in both rows of a pair, the other
+  // with the odd rows'), which stay in the vector ALU instead of going through LDS.
+  typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
   if (LANES >= 32) {
-    // swap the 16-lane halves of each 32-lane group
-    int o = __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401F);
-    v = op(v, __builtin_bit_cast(float, o));
+    const unsigned u = __builtin_bit_cast(unsigned, v);
+    const u32x2 r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    const unsigned even = r.x, odd = r.y;
+    v = op(__builtin_bit_cast(float, even), __builtin_bit_cast(float, odd));
   }
-  if (LANES >= 64) v = op(v, __shfl_xor(v, 32, 64));
+  if (LANES >= 64) {
+    const unsigned u = __builtin_bit_cast(unsigned, v);
+    const u32x2 r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    const unsigned lo = r.x, hi = r.y;
+    v = op(__builtin_bit_cast(float, lo), __builtin_bit_cast(float, hi));
+  }
   return v;
 }
 

@@ -16,6 +16,7 @@ import re
 import shutil
 import subprocess
 import tempfile
+import threading
 from dataclasses import dataclass, field
 
 PKG_ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -122,7 +123,7 @@ def build_kernel(spec: KernelSpec, arch: str | None, path: str, dump_dir: str | 
     generated ISA (`*.s`) for inspection (reference: build.py:73-87)."""
     arch = arch or DEFAULT_ARCH
     os.makedirs(os.path.dirname(os.path.abspath(path)) or ".", exist_ok=True)
-    tmp = f"{path}.tmp{os.getpid()}"
+    tmp = f"{path}.tmp{os.getpid()}_{threading.get_ident()}"
     cmd = compile_command(spec, arch, tmp)
     cwd = None
     if dump_dir:
