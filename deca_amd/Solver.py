@@ -461,7 +461,7 @@ def solve_flash_attn(arch, B: int, H: int, S_q: int, S_kv: int, D: int, type_siz
     """
     from deca_amd.kernels.flash_attn_hip import FAConfig
 
-    if D not in (64, 128, 256):  # the kernel's LDS swizzles need a power-of-two head dim
+    if D % 64 != 0 or D < 64:  # flash_attn_tir.py:70-72
         return []
     cons = _fa_constraints(arch, B, H, S_q, S_kv, D, type_size, max_est_regs)
     return [FAConfig(Br=br, Bc=bc, num_warps=nw, stages=st, pipe=int(pipe))

@@ -87,8 +87,7 @@ constexpr float LOG2E = 1.4426950408889634f;
 constexpr float NEG_INF = -1e30f;
 constexpr float SL2 = static_cast<float>(DECA_SCALE) * LOG2E;
 
-static_assert(D_ == 64 || D_ == 128 || D_ == 256,
-              "head dim: the XOR swizzles of the LDS layouts need a power of two >= 64");
+static_assert(D_ % 64 == 0 && D_ >= 64, "head dim: a multiple of 64 (flash_attn_tir.py:70-72)");
 static_assert(BR % (32 * NW) == 0, "each wave owns a multiple of 32 query rows");
 static_assert(BC % 32 == 0, "BC must be a multiple of 32");
 static_assert(DECA_SQ % BR == 0 && DECA_SKV % BC == 0, "tiles must divide the sequences");
@@ -106,18 +105,30 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef __attribute__((address_space(3))) short4v* lds_s4_ptr;
 typedef __attribute__((address_space(3))) void* lptr;
 
-// LDS layouts.  K tile [BC][D]: 16-byte chunk c of row r sits at chunk slot
-// c ^ ((r / rows_per_window) & mask), so that 16 consecutive rows at one logical
-// chunk land on 16 different bank groups of the 256-byte bank window.  V tile
-// [BC][D]: chunk c of row r sits at c ^ v_swz(r), which puts the 4 key rows that
-// one half of a transposing read touches (64 bytes each) onto the 4 different
-// 64-byte groups of the 256-byte bank window: with 256-byte rows (D = 128) all
-// rows alias and the group is rotated by r % 4; with 128-byte rows (D = 64)
-// rows r and r + 1 already sit in different halves of the window, and rows r
-// and r + 2 are told apart by bit 1 of r.
-constexpr int v_swz(int row) {
-  return CPR >= 16 ? (((row & 3) << 2) & (CPR - 1)) : (((row >> 1) & 1) << 2);
-}
+// LDS layouts.  Rows are D * 2 bytes: a multiple of 256 bytes (the bank window) when
+// D is a multiple of 128, an odd multiple of 128 bytes otherwise (D = 64, 192, 320 ...).
+// K tile [BC][D]: 16-byte chunk c of row r sits at chunk slot c ^ k_swz(r), so that
+// 16 consecutive rows at one logical chunk land on the 16 different 16-byte groups of
+// the window: when all rows alias, the low four chunk bits are XORed with r % 16; when
+// rows r and r + 1 sit in different halves of the window, the low three with
+// (r / 2) % 8.  Only the low bits of c change, so the slot stays inside the row for any
+// number of chunks that is a multiple of 8.  V tile [BC][D]: chunk c of row r sits at
+// c ^ v_swz(r), which puts the 4 key rows that one half of a transposing read touches
+// (64 bytes each) onto the 4 different 64-byte groups of the window: when all rows
+// alias the group is rotated by r % 4, otherwise rows r and r + 2 are told apart by
+// bit 1 of r.
+constexpr bool ROWS_ALIAS = CPR % 16 == 0;
+constexpr int K_XOR_BITS = ROWS_ALIAS ? 4 : 3;
+constexpr int V_XOR_BITS = ROWS_ALIAS ? 2 : 1;  // of the 64-byte group index (chunk bits 2..)
+constexpr int k_swz(int row) { return ROWS_ALIAS ? (row & 15) : ((row >> 1) & 7); }
+constexpr int v_swz(int row) { return ROWS_ALIAS ? ((row & 3) << 2) : (((row >> 1) & 1) << 2); }
+// A read of logical chunk c0 + j (c0 compile-time, j and the swizzle from the lane) is
+// "lane base XOR constant, plus constant": the bits of c0 that the swizzle can reach go
+// into the XOR, the rest is added.
+constexpr unsigned k_xor_const(int c0) { return static_cast<unsigned>(c0 & ((1 << K_XOR_BITS) - 1)) * 16u; }
+constexpr unsigned k_add_const(int c0) { return static_cast<unsigned>(c0 >> K_XOR_BITS << K_XOR_BITS) * 16u; }
+constexpr unsigned v_xor_const(int c0) { return static_cast<unsigned>(c0 & ((4 << V_XOR_BITS) - 1)) * 16u; }
+constexpr unsigned v_add_const(int c0) { return static_cast<unsigned>(c0 >> (2 + V_XOR_BITS) << (2 + V_XOR_BITS)) * 16u; }
 
 // Slices per dispatch group of the causal kernel: the smallest divisor g of the
 // slices of an XCD with g * nq >= 32 workgroups (64 when a slice has 16 or more
@@ -224,9 +235,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
   for (int it = 0; it < KV_IT; ++it) {
     const int sidx = it * NT + tid;
     const int row = sidx / CPR, cs = sidx % CPR;
-    constexpr int ROWS_PER_WINDOW = (16 / CPR) > 0 ? (16 / CPR) : 1;
-    constexpr int MASK = (CPR < 16 ? CPR : 16) - 1;
-    const int ck = cs ^ ((row / ROWS_PER_WINDOW) & MASK);
+    const int ck = cs ^ k_swz(row);
     const int cv = cs ^ v_swz(row);
     k_voff[it] = static_cast<unsigned>(row * D_ + ck * 8) * 2u;
     v_voff[it] = static_cast<unsigned>(row * D_ + cv * 8) * 2u;
@@ -279,14 +288,14 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
   // The swizzles only touch address bits that the loop-varying terms (key block,
   // d block, k-step) either leave alone or toggle as a whole, so every read is
   // "per-lane base XOR compile-time constant, plus an immediate offset".
-  // K: row = kt*32 + lane%32, chunk = (ks*2 + half) ^ swz(row); row bits used by
-  // the swizzle do not depend on kt.
-  constexpr int K_RPW = (16 / CPR) > 0 ? (16 / CPR) : 1;
-  constexpr int K_MASK = (CPR < 16 ? CPR : 16) - 1;
-  const unsigned k_lane_base =
-      static_cast<unsigned>(l32 * CPR + (half ^ ((l32 / K_RPW) & K_MASK))) * 16u;
-  static_assert((32 / K_RPW) % (K_MASK + 1) == 0, "K swizzle must not depend on the key block");
-  // V: row = kk*16 + r*8 + (half*4 + ti/4), chunk = (dt*4 + tb%2*2 + ti%4/2) ^ ((row&3) << 2)
+  // K: row = kt*32 + lane%32, chunk = (ks*2 + half) ^ k_swz(row); the row bits used by
+  // the swizzle do not depend on kt (k_swz has period 16).
+  const unsigned k_lane_base = static_cast<unsigned>(l32 * CPR + (half ^ k_swz(l32))) * 16u;
+  auto k_frag_offset = [&](int ks, int kt) __attribute__((always_inline)) {
+    return (k_lane_base ^ k_xor_const(ks * 2)) + k_add_const(ks * 2) +
+           static_cast<unsigned>(kt * 32 * CPR * 16);
+  };
+  // V: row = kk*16 + r*8 + (half*4 + ti/4), chunk = (dt*4 + tb%2*2 + ti%4/2) ^ v_swz(row)
   const int tb = lane >> 4, ti = lane & 15;
   const int v_row0 = (tb >> 1) * 4 + (ti >> 2);
   const int v_d0 = 16 * (tb & 1) + 4 * (ti & 3);
@@ -294,6 +303,10 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
       v_row0 * CPR * 16 + (((v_d0 >> 3) ^ v_swz(v_row0)) * 16) +
       ((v_d0 >> 2) & 1) * 8);
   static_assert(CPR >= 8, "D >= 64");
+  auto v_frag_offset = [&](int dt, int row0) __attribute__((always_inline)) {
+    return (v_lane_base ^ v_xor_const(dt * 4)) + v_add_const(dt * 4) +
+           static_cast<unsigned>(row0 * CPR * 16);
+  };
   // ---- the three phases of one KV step ----------------------------------------------------
   // S^T = K Q^T for the tile in K slot `kslot`
   auto compute_s = [&](floatx16 (&s_acc)[KT][MQ], int kslot) __attribute__((always_inline)) {
@@ -308,8 +321,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
     for (int ks = 0; ks < DK; ++ks) {
 #pragma unroll
       for (int kt = 0; kt < KT; ++kt) {
-        const half8 kf = *reinterpret_cast<const half8*>(
-            k_lds + ((k_lane_base ^ static_cast<unsigned>(ks * 32)) + kt * 32 * CPR * 16));
+        const half8 kf = *reinterpret_cast<const half8*>(k_lds + k_frag_offset(ks, kt));
 #pragma unroll
         for (int mq = 0; mq < MQ; ++mq)
           s_acc[kt][mq] =
@@ -413,9 +425,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
         half4 h[2];
 #pragma unroll
         for (int r = 0; r < 2; ++r) {
-          const unsigned char* p =
-              v_lds + ((v_lane_base ^ static_cast<unsigned>((dt * 4 * 16) & (CPR * 16 - 1))) +
-                       (kk * 16 + r * 8) * CPR * 16);
+          const unsigned char* p = v_lds + v_frag_offset(dt, kk * 16 + r * 8);
           h[r] = __builtin_bit_cast(half4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4_ptr)(p)));
         }
         const half8 vf = __builtin_shufflevector(h[0], h[1], 0, 1, 2, 3, 4, 5, 6, 7);
@@ -533,8 +543,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
                             half8 (&pf)[KK][MQ], int kslot) {
     const unsigned char* k_lds = lds + kslot * TILE_BYTES;
     constexpr int STEPS = DK * KT;
-    constexpr int EPS_ = (KT * 16) / STEPS;  // scores of the current tile per step and q tile
-    static_assert((KT * 16) % STEPS == 0 && EPS_ >= 1, "scores must divide over the steps");
+    constexpr int NE_ = KT * 16;  // scores of the current tile per lane and q tile, dealt over the steps
     const floatx16 zero = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f,
                            0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
     float sum[MQ];
@@ -547,8 +556,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
       const half8 kf = kf_next;
       if (step + 1 < STEPS) {
         const int ks1 = (step + 1) / KT, kt1 = (step + 1) % KT;
-        kf_next = *reinterpret_cast<const half8*>(
-            k_lds + ((k_lane_base ^ static_cast<unsigned>(ks1 * 32)) + kt1 * 32 * CPR * 16));
+        kf_next = *reinterpret_cast<const half8*>(k_lds + k_frag_offset(ks1, kt1));
       }
 #pragma unroll
       for (int mq = 0; mq < MQ; ++mq)
@@ -557,8 +565,8 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
 #pragma unroll
       for (int mq = 0; mq < MQ; ++mq)
 #pragma unroll
-        for (int i = 0; i < EPS_; ++i) {
-          const int lin = step * EPS_ + i, ct = lin / 16, ce = lin % 16;
+        for (int lin = step * NE_ / STEPS; lin < (step + 1) * NE_ / STEPS; ++lin) {
+          const int ct = lin / 16, ce = lin % 16;
           const float p =
               __builtin_amdgcn_exp2f(__builtin_fmaf(s_cur[ct][mq][ce], SL2, -msl[mq]));
           s_cur[ct][mq][ce] = p;
@@ -636,15 +644,13 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
       constexpr int t = decltype(tc)::value;
       if constexpr (t < S_SLOTS) {
         constexpr int pr = t / (2 * DK), r = t % (2 * DK), ks = r / 2, kt = 2 * pr + r % 2;
-        return *reinterpret_cast<const half8*>(
-            k_lds + ((k_lane_base ^ static_cast<unsigned>(ks * 32)) + kt * 32 * CPR * 16));
+        return *reinterpret_cast<const half8*>(k_lds + k_frag_offset(ks, kt));
       } else {
         constexpr int u = t - S_SLOTS, kk = u / DT, dt = u % DT;
-        const unsigned base = v_lane_base ^ static_cast<unsigned>((dt * 4 * 16) & (CPR * 16 - 1));
         const half4 h0 = __builtin_bit_cast(half4, __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (lds_s4_ptr)(v_lds + (base + (kk * 16) * CPR * 16))));
+            (lds_s4_ptr)(v_lds + v_frag_offset(dt, kk * 16))));
         const half4 h1 = __builtin_bit_cast(half4, __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (lds_s4_ptr)(v_lds + (base + (kk * 16 + 8) * CPR * 16))));
+            (lds_s4_ptr)(v_lds + v_frag_offset(dt, kk * 16 + 8))));
         return __builtin_shufflevector(h0, h1, 0, 1, 2, 3, 4, 5, 6, 7);
       }
     };

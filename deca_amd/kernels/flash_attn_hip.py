@@ -132,9 +132,9 @@ def slot_schedule_ok(Bc: int, D: int) -> bool:
 
 
 def check_config(cfg: FAConfig, S_q: int, S_kv: int, D: int) -> None:
-    # reference: D % 64 == 0 (flash_attn_tir.py:71); the XOR swizzles of the LDS layouts here
-    # need a power of two as well
-    assert D in (64, 128, 256), "head dim must be 64, 128 or 256"
+    # as the reference (flash_attn_tir.py:70-72); the LDS swizzles only touch the low chunk
+    # bits of a row, so any row of a multiple of 8 chunks works
+    assert D % 64 == 0 and D >= 64, "head dim must be a multiple of 64"
     assert cfg.Br % (32 * cfg.num_warps) == 0
     assert cfg.Bc % 32 == 0
     assert S_q % cfg.Br == 0 and S_kv % cfg.Bc == 0

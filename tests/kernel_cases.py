@@ -170,6 +170,14 @@ FA_CASES = [
     # key tiles wider than the query tiles
     (1, 2, 512, 512, 64, True, FAConfig(128, 128, 4, 2, pipe=2)),
     (1, 2, 1024, 1024, 64, True, FAConfig(64, 128, 2, 2, pipe=2)),
+    # head dims that are multiples of 64 but no powers of two: full, causal, the three loops
+    (1, 2, 256, 256, 192, False, FAConfig(128, 64, 4, 2)),
+    (1, 2, 256, 256, 192, True, FAConfig(128, 64, 4, 2)),
+    (1, 2, 256, 384, 192, False, FAConfig(64, 32, 2, 1)),
+    (1, 2, 512, 512, 192, True, FAConfig(128, 64, 4, 2, pipe=1)),
+    (1, 2, 512, 512, 192, False, FAConfig(128, 64, 4, 2, pipe=2)),
+    (1, 2, 512, 512, 192, True, FAConfig(128, 64, 4, 2, pipe=2)),
+    (1, 1, 256, 256, 320, True, FAConfig(32, 32, 1, 2)),
 ]
 
 FA_FULL = [

@@ -235,15 +235,16 @@ def test_kernels_are_compiled_for_the_occupancy_the_estimates_allow():
 
 
 def test_flash_attn_head_dims():
-    """64, 128 and 256 are supported; other multiples of 64 (which the reference accepts,
-    flash_attn_tir.py:71) have no LDS layout here and yield no config instead of a bad one."""
-    assert Solver.solve_flash_attn(ARCH, 4, 16, 2048, 2048, 192) == []
-    wide = Solver.solve_flash_attn(ARCH, 4, 16, 2048, 2048, 256)
-    assert wide
-    for cfg in wide:
-        fa.check_config(cfg, 2048, 2048, 256)
+    """Every multiple of 64 is supported, as in the reference (flash_attn_tir.py:70-72);
+    anything else yields no config instead of a bad one."""
+    for D in (192, 256, 320):
+        wide = Solver.solve_flash_attn(ARCH, 4, 16, 2048, 2048, D)
+        assert wide
+        for cfg in wide:
+            fa.check_config(cfg, 2048, 2048, D)
+    assert Solver.solve_flash_attn(ARCH, 4, 16, 2048, 2048, 96) == []
     with pytest.raises(AssertionError):
-        fa.check_config(fa.FAConfig(128, 64, 4, 2), 2048, 2048, 192)
+        fa.check_config(fa.FAConfig(128, 64, 4, 2), 2048, 2048, 96)
 
 
 def test_gemm_tail_split_is_offered_where_a_partial_wave_remains():
