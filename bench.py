@@ -297,6 +297,9 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default=DEFAULT_WORKLOAD)
+    ap.add_argument("--kernel-config", default=None, metavar="TEXT",
+                    help="time this kernel configuration (in the form the records print) for "
+                         "--workload instead of its stored winner; implies --no-extra")
     ap.add_argument("--no-extra", action="store_true", help="only the headline workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     args = ap.parse_args()
@@ -310,6 +313,13 @@ def main():
         print("bench.py needs a GPU (the kernels have no host path)", file=sys.stderr)
         sys.exit(1)
     wls = workloads()
+    if args.kernel_config:
+        from deca_amd import tuned
+
+        wl = wls[args.workload]
+        op = {"gemm": "GEMM", "fa": "flash_attn"}.get(wl["kind"]) or wl["op"]
+        wl["cfg"] = tuned.parse_config(op, args.kernel_config)
+        args.no_extra = True
     head = run(wls[args.workload], args.steps, args.warmup, not args.no_cpu)
     out = {
         "metric": head["metric"],

@@ -389,6 +389,7 @@ FA_DOMAINS = {
     "nw": (1, 2, 4, 8),
     "st": (1, 2),
     "pipe": (0, 1, 2),
+    "mfma": (32, 16),  # 16: v_mfma_f32_16x16x32 tiles (plain and slot loop)
 }
 
 
@@ -400,9 +401,10 @@ def _fa_constraints(arch, B: int, H: int, S_q: int, S_kv: int, D: int, type_size
     simds = arch.simds_per_cu
 
     def build(o, v):
-        br, bc, nw, st, pipe = (v[k] for k in FA_DOMAINS)
+        br, bc, nw, st, pipe, mfma = (v[k] for k in FA_DOMAINS)
         c = o.const
-        slot_bcs = [b for b in FA_DOMAINS["bc"] if slot_schedule_ok(b, D)] or [0]
+        slot_bcs = {m: [b for b in FA_DOMAINS["bc"] if slot_schedule_ok(b, D, m)] or [0]
+                    for m in FA_DOMAINS["mfma"]}
         threads = nw * wave
         cpr = D // 8
         out = [
@@ -421,7 +423,10 @@ def _fa_constraints(arch, B: int, H: int, S_q: int, S_kv: int, D: int, type_size
             # the software-pipelined loop runs one K tile ahead: two slots, two tiles
             o.implies(o.uge(pipe, c(1)), o.all_of(o.eq(st, c(2)), o.uge(o.udiv(c(S_kv), bc), c(2)))),
             # the slot-interleaved loop issues the S^T chains in pairs of 32-key blocks
-            o.implies(o.eq(pipe, c(2)), o.any_of(*[o.eq(bc, c(b)) for b in slot_bcs])),
+            *[o.implies(o.all_of(o.eq(pipe, c(2)), o.eq(mfma, c(m))),
+                        o.any_of(*[o.eq(bc, c(b)) for b in slot_bcs[m]])) for m in slot_bcs],
+            # the 16x16x32 form exists for the plain and the slot loop
+            o.implies(o.eq(mfma, c(16)), o.any_of(o.eq(pipe, c(0)), o.eq(pipe, c(2)))),
         ]
         # registers: O^T accumulator + S^T accumulator + P + Q fragments + K/V fragments
         mq = o.udiv(br, nw * 32)
@@ -464,5 +469,5 @@ def solve_flash_attn(arch, B: int, H: int, S_q: int, S_kv: int, D: int, type_siz
     if D % 64 != 0 or D < 64:  # flash_attn_tir.py:70-72
         return []
     cons = _fa_constraints(arch, B, H, S_q, S_kv, D, type_size, max_est_regs)
-    return [FAConfig(Br=br, Bc=bc, num_warps=nw, stages=st, pipe=int(pipe))
-            for br, bc, nw, st, pipe in _enumerate(FA_DOMAINS, cons, count, backend)]
+    return [FAConfig(Br=br, Bc=bc, num_warps=nw, stages=st, pipe=int(pipe), mfma=mfma)
+            for br, bc, nw, st, pipe, mfma in _enumerate(FA_DOMAINS, cons, count, backend)]

@@ -72,11 +72,35 @@
 
 constexpr int NT = NW * 64;
 constexpr int WQ = BR / NW;       // query rows per wave
+#ifndef DECA_MFMA16
+#define DECA_MFMA16 0  // 1: v_mfma_f32_16x16x32_f16 tiles (plain loop only) instead of 32x32x16
+#endif
+#if DECA_MFMA16
+// 16 x 16 accumulator tiles, k-steps of 32.  A lane holds ONE query column (lane % 16)
+// and 4 key rows (4 * (lane / 16) .. +3) per 16-key block; the four 16-lane groups of a
+// query are reduced with two row swaps.  P^T for one O^T step (32 keys) is the pair of
+// key blocks 2kk, 2kk + 1: operand k-index 8g + i is key 4g + i of block 2kk (i < 4) or
+// key 4g + i - 4 of block 2kk + 1, and V^T is read in the same key order.
+constexpr int TQ = 16;            // queries per MFMA tile
+constexpr int MQ = WQ / 16;       // query tiles per wave
+constexpr int KT = BC / 16;       // 16-key blocks per step
+constexpr int DK = D_ / 32;       // k-steps of S^T = K Q^T
+constexpr int DT = D_ / 16;       // 16-d blocks of O^T
+constexpr int KK = BC / 32;       // k-steps of O^T = V^T P^T
+constexpr int ACC_N = 4;
+constexpr int K_CHUNKS_PER_STEP = 4, V_CHUNKS_PER_BLOCK = 2;
+static_assert(DECA_PIPE != 1, "the 16x16x32 form is written for the plain and the slot loop");
+static_assert(BC % 32 == 0 && WQ % 16 == 0, "tiles of the 16x16x32 form");
+#else
+constexpr int TQ = 32;
 constexpr int MQ = WQ / 32;       // 32-query MFMA tiles per wave
 constexpr int KT = BC / 32;       // 32-key blocks per step (S^T row tiles)
 constexpr int DK = D_ / 16;       // k-steps of S^T = K Q^T
 constexpr int DT = D_ / 32;       // 32-d blocks of O^T
 constexpr int KK = BC / 16;       // k-steps of O^T = V^T P^T
+constexpr int ACC_N = 16;
+constexpr int K_CHUNKS_PER_STEP = 2, V_CHUNKS_PER_BLOCK = 4;
+#endif
 constexpr int CPR = D_ / 8;       // 16-byte chunks per K/V row
 constexpr int TILE_CHUNKS = BC * CPR;
 constexpr int TILE_BYTES = TILE_CHUNKS * 16;
@@ -102,7 +126,18 @@ typedef _Float16 half4 __attribute__((ext_vector_type(4)));
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef short short4v __attribute__((ext_vector_type(4)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+#if DECA_MFMA16
+typedef floatx4 acc_t;
+#else
+typedef floatx16 acc_t;
+#endif
 typedef __attribute__((address_space(3))) short4v* lds_s4_ptr;
+#if DECA_MFMA16
+#define DECA_MFMA __builtin_amdgcn_mfma_f32_16x16x32_f16
+#else
+#define DECA_MFMA __builtin_amdgcn_mfma_f32_32x32x16_f16
+#endif
 typedef __attribute__((address_space(3))) void* lptr;
 
 // LDS layouts.  Rows are D * 2 bytes: a multiple of 256 bytes (the bank window) when
@@ -121,7 +156,15 @@ constexpr bool ROWS_ALIAS = CPR % 16 == 0;
 constexpr int K_XOR_BITS = ROWS_ALIAS ? 4 : 3;
 constexpr int V_XOR_BITS = ROWS_ALIAS ? 2 : 1;  // of the 64-byte group index (chunk bits 2..)
 constexpr int k_swz(int row) { return ROWS_ALIAS ? (row & 15) : ((row >> 1) & 7); }
+#if DECA_MFMA16
+// (the two 16-lane blocks of a half-wave read rows r and r + 4 of the same 32-byte column
+// range: bit 2 of r moves them to different halves of the 64-byte group)
+constexpr int v_swz(int row) {
+  return (ROWS_ALIAS ? ((row & 3) << 2) : (((row >> 1) & 1) << 2)) | (((row >> 2) & 1) << 1);
+}
+#else
 constexpr int v_swz(int row) { return ROWS_ALIAS ? ((row & 3) << 2) : (((row >> 1) & 1) << 2); }
+#endif
 // A read of logical chunk c0 + j (c0 compile-time, j and the swizzle from the lane) is
 // "lane base XOR constant, plus constant": the bits of c0 that the swizzle can reach go
 // into the XOR, the rest is added.
@@ -171,6 +214,33 @@ __device__ __forceinline__ float sum_halves(float x) {
   float a, b;
   both_halves(x, a, b);
   return a + b;
+}
+// The same for the 16-lane rows l and l ^ 16 (v_permlane16_swap).
+__device__ __forceinline__ void both_rows(float x, float& even, float& odd) {
+  typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+  const unsigned u = __builtin_bit_cast(unsigned, x);
+  const u32x2 r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  const unsigned e = r.x, o = r.y;
+  even = __builtin_bit_cast(float, e);
+  odd = __builtin_bit_cast(float, o);
+}
+// Reduction over the lanes that hold one query column: lanes l and l ^ 32 in the 32x32x16
+// form, the four lanes l % 16 + {0, 16, 32, 48} in the 16x16x32 form.
+__device__ __forceinline__ float max_over_query(float x) {
+#if DECA_MFMA16
+  float a, b;
+  both_rows(x, a, b);
+  x = fmaxf(a, b);
+#endif
+  return max_halves(x);
+}
+__device__ __forceinline__ float sum_over_query(float x) {
+#if DECA_MFMA16
+  float a, b;
+  both_rows(x, a, b);
+  x = a + b;
+#endif
+  return sum_halves(x);
 }
 
 #define DECA_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (((n) >> 4) << 14) | 0x0F70)
@@ -263,20 +333,30 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
 
   // ---- Q fragments: VGPR resident for the whole kernel ----------------------------
   // lane (q = lane % 32, half): 8 consecutive d at ks * 16 + half * 8
+  // (16x16x32: q = lane % 16, 8 consecutive d at ks * 32 + (lane / 16) * 8)
+  const int tb = lane >> 4, ti = lane & 15;
+#if DECA_MFMA16
+  const int lq = ti;      // query column of this lane inside a query tile
+  const int lg = tb;      // which quarter of a k-step / of a key block this lane holds
+#else
+  const int lq = l32;
+  const int lg = half;
+#endif
   half8 qf[MQ][DK];
 #pragma unroll
   for (int mq = 0; mq < MQ; ++mq)
 #pragma unroll
     for (int ks = 0; ks < DK; ++ks)
-      qf[mq][ks] = *reinterpret_cast<const half8*>(q_base + (mq * 32 + l32) * D_ + ks * 16 + half * 8);
+      qf[mq][ks] = *reinterpret_cast<const half8*>(
+          q_base + (mq * TQ + lq) * D_ + ks * (K_CHUNKS_PER_STEP * 8) + lg * 8);
 
-  floatx16 o_acc[DT][MQ];
+  acc_t o_acc[DT][MQ];
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
     for (int mq = 0; mq < MQ; ++mq)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) o_acc[dt][mq][e] = 0.0f;
+      for (int e = 0; e < ACC_N; ++e) o_acc[dt][mq][e] = 0.0f;
   float m_i[MQ], l_i[MQ];
 #pragma unroll
   for (int mq = 0; mq < MQ; ++mq) {
@@ -290,33 +370,39 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
   // "per-lane base XOR compile-time constant, plus an immediate offset".
   // K: row = kt*32 + lane%32, chunk = (ks*2 + half) ^ k_swz(row); the row bits used by
   // the swizzle do not depend on kt (k_swz has period 16).
-  const unsigned k_lane_base = static_cast<unsigned>(l32 * CPR + (half ^ k_swz(l32))) * 16u;
+  // (16x16x32: row = kt*16 + lane%16, chunk = (ks*4 + lane/16) ^ k_swz(row))
+  const unsigned k_lane_base = static_cast<unsigned>(lq * CPR + (lg ^ k_swz(lq))) * 16u;
   auto k_frag_offset = [&](int ks, int kt) __attribute__((always_inline)) {
-    return (k_lane_base ^ k_xor_const(ks * 2)) + k_add_const(ks * 2) +
-           static_cast<unsigned>(kt * 32 * CPR * 16);
+    return (k_lane_base ^ k_xor_const(ks * K_CHUNKS_PER_STEP)) + k_add_const(ks * K_CHUNKS_PER_STEP) +
+           static_cast<unsigned>(kt * TQ * CPR * 16);
   };
   // V: row = kk*16 + r*8 + (half*4 + ti/4), chunk = (dt*4 + tb%2*2 + ti%4/2) ^ v_swz(row)
-  const int tb = lane >> 4, ti = lane & 15;
+  // (16x16x32: row = block*16 + (lane/16)*4 + ti/4, chunk = (dt*2 + ti%4/2) ^ v_swz(row))
+#if DECA_MFMA16
+  const int v_row0 = tb * 4 + (ti >> 2);
+  const int v_d0 = 4 * (ti & 3);
+#else
   const int v_row0 = (tb >> 1) * 4 + (ti >> 2);
   const int v_d0 = 16 * (tb & 1) + 4 * (ti & 3);
+#endif
   const unsigned v_lane_base = static_cast<unsigned>(
       v_row0 * CPR * 16 + (((v_d0 >> 3) ^ v_swz(v_row0)) * 16) +
       ((v_d0 >> 2) & 1) * 8);
   static_assert(CPR >= 8, "D >= 64");
   auto v_frag_offset = [&](int dt, int row0) __attribute__((always_inline)) {
-    return (v_lane_base ^ v_xor_const(dt * 4)) + v_add_const(dt * 4) +
+    return (v_lane_base ^ v_xor_const(dt * V_CHUNKS_PER_BLOCK)) + v_add_const(dt * V_CHUNKS_PER_BLOCK) +
            static_cast<unsigned>(row0 * CPR * 16);
   };
   // ---- the three phases of one KV step ----------------------------------------------------
   // S^T = K Q^T for the tile in K slot `kslot`
-  auto compute_s = [&](floatx16 (&s_acc)[KT][MQ], int kslot) __attribute__((always_inline)) {
+  auto compute_s = [&](acc_t (&s_acc)[KT][MQ], int kslot) __attribute__((always_inline)) {
     const unsigned char* k_lds = lds + kslot * TILE_BYTES;
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
       for (int mq = 0; mq < MQ; ++mq)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) s_acc[kt][mq][e] = 0.0f;
+        for (int e = 0; e < ACC_N; ++e) s_acc[kt][mq][e] = 0.0f;
 #pragma unroll
     for (int ks = 0; ks < DK; ++ks) {
 #pragma unroll
@@ -324,25 +410,28 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
         const half8 kf = *reinterpret_cast<const half8*>(k_lds + k_frag_offset(ks, kt));
 #pragma unroll
         for (int mq = 0; mq < MQ; ++mq)
-          s_acc[kt][mq] =
-              __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[mq][ks], s_acc[kt][mq], 0, 0, 0);
+          s_acc[kt][mq] = DECA_MFMA(kf, qf[mq][ks], s_acc[kt][mq], 0, 0, 0);
       }
     }
   };
   // Causal mask of tile j.  Only tiles crossing the diagonal need it; every
   // query sees key 0 in tile 0, so its running max is finite before a fully
   // masked block shows up.
-  auto mask_s = [&](floatx16 (&s_acc)[KT][MQ], int j) __attribute__((always_inline)) {
+  auto mask_s = [&](acc_t (&s_acc)[KT][MQ], int j) __attribute__((always_inline)) {
 #if DECA_CAUSAL
     if ((j + 1) * BC - 1 > qt * BR + wave * WQ) {
 #pragma unroll
       for (int mq = 0; mq < MQ; ++mq) {
-        const int q_idx = qt * BR + wave * WQ + mq * 32 + l32;
+        const int q_idx = qt * BR + wave * WQ + mq * TQ + lq;
 #pragma unroll
         for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
-          for (int e = 0; e < 16; ++e) {
+          for (int e = 0; e < ACC_N; ++e) {
+#if DECA_MFMA16
+            const int kv_idx = j * BC + kt * 16 + lg * 4 + e;
+#else
             const int kv_idx = j * BC + kt * 32 + (e >> 2) * 8 + half * 4 + (e & 3);
+#endif
             if (kv_idx > q_idx) s_acc[kt][mq][e] = NEG_INF;
           }
       }
@@ -368,7 +457,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
   // Online softmax of one tile: one query column per lane.  Leaves P^T (fp16,
   // already in operand order) in `pf` and rescales O^T when a running max moved
   // (skipped otherwise: multiplying by 1 is exact).
-  auto softmax = [&](floatx16 (&s_acc)[KT][MQ], half8 (&pf)[KK][MQ]) __attribute__((always_inline)) {
+  auto softmax = [&](acc_t (&s_acc)[KT][MQ], half8 (&pf)[KK][MQ]) __attribute__((always_inline)) {
     float alpha[MQ];
 #pragma unroll
     for (int mq = 0; mq < MQ; ++mq) {
@@ -376,8 +465,8 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
 #pragma unroll
       for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) mx = fmaxf(mx, s_acc[kt][mq][e]);
-      mx = max_halves(mx);
+        for (int e = 0; e < ACC_N; ++e) mx = fmaxf(mx, s_acc[kt][mq][e]);
+      mx = max_over_query(mx);
       const float m_new = lazy_max(m_i[mq], mx);
       alpha[mq] = __builtin_amdgcn_exp2f((m_i[mq] - m_new) * SL2);
       m_i[mq] = m_new;
@@ -386,11 +475,12 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
 #pragma unroll
       for (int kt = 0; kt < KT; ++kt) {
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
+        for (int e = 0; e < ACC_N; ++e) {
           const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s_acc[kt][mq][e], SL2, -msl));
           s_acc[kt][mq][e] = p;
           sum += p;
         }
+#if !DECA_MFMA16
 #pragma unroll
         for (int hh = 0; hh < 2; ++hh) {
           half8 h;
@@ -398,7 +488,20 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
           for (int e = 0; e < 8; ++e) h[e] = static_cast<_Float16>(s_acc[kt][mq][hh * 8 + e]);
           pf[kt * 2 + hh][mq] = h;
         }
+#endif
       }
+#if DECA_MFMA16
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk) {
+        half8 h;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          h[e] = static_cast<_Float16>(s_acc[2 * kk][mq][e]);
+          h[4 + e] = static_cast<_Float16>(s_acc[2 * kk + 1][mq][e]);
+        }
+        pf[kk][mq] = h;
+      }
+#endif
       l_i[mq] = l_i[mq] * alpha[mq] + sum;
     }
     bool moved = false;
@@ -410,7 +513,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
 #pragma unroll
         for (int mq = 0; mq < MQ; ++mq)
 #pragma unroll
-          for (int e = 0; e < 16; ++e) o_acc[dt][mq][e] *= alpha[mq];
+          for (int e = 0; e < ACC_N; ++e) o_acc[dt][mq][e] *= alpha[mq];
     }
   };
   // O^T += V^T P^T for the tile in V slot `vslot`.  k-slot (half, e) of step kk
@@ -425,14 +528,17 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
         half4 h[2];
 #pragma unroll
         for (int r = 0; r < 2; ++r) {
+#if DECA_MFMA16
+          const unsigned char* p = v_lds + v_frag_offset(dt, (2 * kk + r) * 16);
+#else
           const unsigned char* p = v_lds + v_frag_offset(dt, kk * 16 + r * 8);
+#endif
           h[r] = __builtin_bit_cast(half4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4_ptr)(p)));
         }
         const half8 vf = __builtin_shufflevector(h[0], h[1], 0, 1, 2, 3, 4, 5, 6, 7);
 #pragma unroll
         for (int mq = 0; mq < MQ; ++mq)
-          o_acc[dt][mq] =
-              __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf[kk][mq], o_acc[dt][mq], 0, 0, 0);
+          o_acc[dt][mq] = DECA_MFMA(vf, pf[kk][mq], o_acc[dt][mq], 0, 0, 0);
       }
     }
   };
@@ -461,7 +567,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
     // made the kernel slower.)
     if (j * BC > qt * BR + wave_u * WQ + WQ - 1) return;
 #endif
-    floatx16 s_acc[KT][MQ];
+    acc_t s_acc[KT][MQ];
     half8 pf[KK][MQ];
     compute_s(s_acc, slot);
     mask_s(s_acc, j);
@@ -483,15 +589,15 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
   static_assert(STAGES == 2, "the pipelined loop uses two K and two V slots");
   float alpha[MQ], msl[MQ];
   // m' = max(m, rowmax S); alpha = exp2((m - m') * sl2); msl = m' * sl2
-  auto row_stats = [&](const floatx16 (&s_acc)[KT][MQ]) __attribute__((always_inline)) {
+  auto row_stats = [&](const acc_t (&s_acc)[KT][MQ]) __attribute__((always_inline)) {
 #pragma unroll
     for (int mq = 0; mq < MQ; ++mq) {
       float mx = s_acc[0][mq][0];
 #pragma unroll
       for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) mx = fmaxf(mx, s_acc[kt][mq][e]);
-      mx = max_halves(mx);
+        for (int e = 0; e < ACC_N; ++e) mx = fmaxf(mx, s_acc[kt][mq][e]);
+      mx = max_over_query(mx);
       const float m_new = lazy_max(m_i[mq], mx);
       alpha[mq] = __builtin_amdgcn_exp2f((m_i[mq] - m_new) * SL2);
       m_i[mq] = m_new;
@@ -508,29 +614,30 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
 #pragma unroll
         for (int mq = 0; mq < MQ; ++mq)
 #pragma unroll
-          for (int e = 0; e < 16; ++e) o_acc[dt][mq][e] *= alpha[mq];
+          for (int e = 0; e < ACC_N; ++e) o_acc[dt][mq][e] *= alpha[mq];
     }
   };
-  // p = exp2(S * sl2 - msl); l = l * alpha + sum p; P = fp16(p) in operand order
-  auto exp_and_pack = [&](floatx16 (&s_acc)[KT][MQ], half8 (&pf)[KK][MQ]) __attribute__((always_inline)) {
+  // p = exp2(S * sl2 - msl); l = l * alpha + sum p; P = fp16(p) in operand order: score
+  // number n = kt * ACC_N + e of a lane is element n % 8 of the operand of k-step n / 8
+  auto exp_and_pack = [&](acc_t (&s_acc)[KT][MQ], half8 (&pf)[KK][MQ]) __attribute__((always_inline)) {
 #pragma unroll
     for (int mq = 0; mq < MQ; ++mq) {
       float sum = 0.0f;
 #pragma unroll
-      for (int kt = 0; kt < KT; ++kt) {
+      for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
+        for (int e = 0; e < ACC_N; ++e) {
           const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s_acc[kt][mq][e], SL2, -msl[mq]));
           s_acc[kt][mq][e] = p;
           sum += p;
         }
 #pragma unroll
-        for (int hh = 0; hh < 2; ++hh) {
-          half8 h;
+      for (int kk = 0; kk < KK; ++kk) {
+        half8 h;
 #pragma unroll
-          for (int e = 0; e < 8; ++e) h[e] = static_cast<_Float16>(s_acc[kt][mq][hh * 8 + e]);
-          pf[kt * 2 + hh][mq] = h;
-        }
+        for (int e = 0; e < 8; ++e)
+          h[e] = static_cast<_Float16>(s_acc[(kk * 8 + e) / ACC_N][mq][(kk * 8 + e) % ACC_N]);
+        pf[kk][mq] = h;
       }
       l_i[mq] = l_i[mq] * alpha[mq] + sum;
     }
@@ -539,6 +646,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
   // current one: after the MFMAs of step (ks, kt) a fixed share of the current
   // tile's scores is exponentiated, and nothing is allowed to move across the
   // step boundary, so the matrix pipe and the vector ALU stay busy together.
+#if DECA_PIPE == 1
   auto s_next_and_exp = [&](floatx16 (&s_nxt)[KT][MQ], floatx16 (&s_cur)[KT][MQ],
                             half8 (&pf)[KK][MQ], int kslot) {
     const unsigned char* k_lds = lds + kslot * TILE_BYTES;
@@ -584,6 +692,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
 #pragma unroll
     for (int mq = 0; mq < MQ; ++mq) l_i[mq] = l_i[mq] * alpha[mq] + sum[mq];
   };
+#endif
 
 #if DECA_PIPE == 2
   // ---- slot-interleaved loop ----------------------------------------------------------------
@@ -599,8 +708,8 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
   static_assert(STAGES == 2, "two K and two V slots");
   static_assert(KT % 2 == 0, "S^T chains are issued in pairs");
   constexpr int S_SLOTS = KT * DK, PV_SLOTS = KK * DT, NS = S_SLOTS + PV_SLOTS;
-  constexpr int NE = KT * 16;             // scores per lane and query tile
-  constexpr int NM = KT * 8;              // max3 operations of the running max
+  constexpr int NE = KT * ACC_N;          // scores per lane and query tile
+  constexpr int NM = NE / 2;              // max3 operations of the running max
   constexpr int PVM = PV_SLOTS - 1;       // O^T slots that carry the running max
   struct Sched {
     static constexpr int ne_s() { return NE * 5 / 8; }          // exponentials under the S^T slots
@@ -625,7 +734,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
   auto finish_stats = [&](float (&mx)[MQ]) __attribute__((always_inline)) {
 #pragma unroll
     for (int mq = 0; mq < MQ; ++mq) {
-      const float mxx = max_halves(mx[mq]);
+      const float mxx = max_over_query(mx[mq]);
       const float m_new = lazy_max(m_i[mq], mxx);
       alpha[mq] = __builtin_amdgcn_exp2f((m_i[mq] - m_new) * SL2);
       m_i[mq] = m_new;
@@ -633,12 +742,14 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
     }
   };
   half2v pf2[KK][MQ][4];
-  auto fused = [&](auto v_slot, floatx16 (&sc)[KT][MQ], floatx16 (&sn)[KT][MQ]) __attribute__((always_inline)) {
+  // Score number n of a lane and query tile lives in accumulator n / ACC_N, register n % ACC_N.
+  auto fused = [&](auto v_slot, acc_t (&sc)[KT][MQ], acc_t (&sn)[KT][MQ]) __attribute__((always_inline)) {
     constexpr int VSLOT = decltype(v_slot)::value;  // V_j; K_{j+1} is in the other K slot
     const unsigned char* k_lds = lds + (VSLOT ^ 1) * TILE_BYTES;
     const unsigned char* v_lds = lds + (STAGES + VSLOT) * TILE_BYTES;
-    const floatx16 zero = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f,
-                           0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    acc_t zero;
+#pragma unroll
+    for (int e = 0; e < ACC_N; ++e) zero[e] = 0.0f;
     // slot t < S_SLOTS: pair p of key blocks, k-step ks, block kt; else k-step kk, d block dt
     auto read_frag = [&](auto tc) __attribute__((always_inline)) -> half8 {
       constexpr int t = decltype(tc)::value;
@@ -647,10 +758,11 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
         return *reinterpret_cast<const half8*>(k_lds + k_frag_offset(ks, kt));
       } else {
         constexpr int u = t - S_SLOTS, kk = u / DT, dt = u % DT;
+        constexpr int V_ROW_STEP = DECA_MFMA16 ? 16 : 8;  // the two key quartets of a lane
         const half4 h0 = __builtin_bit_cast(half4, __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (lds_s4_ptr)(v_lds + v_frag_offset(dt, kk * 16))));
+            (lds_s4_ptr)(v_lds + v_frag_offset(dt, kk * 2 * V_ROW_STEP))));
         const half4 h1 = __builtin_bit_cast(half4, __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (lds_s4_ptr)(v_lds + v_frag_offset(dt, kk * 16 + 8))));
+            (lds_s4_ptr)(v_lds + v_frag_offset(dt, kk * 2 * V_ROW_STEP + V_ROW_STEP))));
         return __builtin_shufflevector(h0, h1, 0, 1, 2, 3, 4, 5, 6, 7);
       }
     };
@@ -671,11 +783,11 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
         // row sum and packing of what slot t-1 exponentiated
         static_for<Sched::e_end(t - 1) - Sched::e_end(t - 2)>([&](auto ic) {
           constexpr int e = Sched::e_end(t - 2) + decltype(ic)::value;
-          sum[mq][e & 1] += sc[e / 16][mq][e % 16];
+          sum[mq][e & 1] += sc[e / ACC_N][mq][e % ACC_N];
           pin(sum[mq][e & 1]);
           if constexpr (e & 1) {
             typedef float float2v __attribute__((ext_vector_type(2)));
-            const float2v pr = {sc[e / 16][mq][e % 16 - 1], sc[e / 16][mq][e % 16]};
+            const float2v pr = {sc[e / ACC_N][mq][e % ACC_N - 1], sc[e / ACC_N][mq][e % ACC_N]};
             unsigned packed = __builtin_bit_cast(unsigned, __builtin_convertvector(pr, half2v));
             pin(packed);
             pf2[e / 8][mq][(e % 8) / 2] = __builtin_bit_cast(half2v, packed);
@@ -683,11 +795,11 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
         });
         static_for<Sched::e_end(t) - Sched::e_end(t - 1)>([&](auto ic) {
           constexpr int e = Sched::e_end(t - 1) + decltype(ic)::value;
-          sc[e / 16][mq][e % 16] = __builtin_amdgcn_exp2f(sc[e / 16][mq][e % 16]);
+          sc[e / ACC_N][mq][e % ACC_N] = __builtin_amdgcn_exp2f(sc[e / ACC_N][mq][e % ACC_N]);
         });
         static_for<Sched::e_end(t + 1) - Sched::e_end(t)>([&](auto ic) {
           constexpr int e = Sched::e_end(t) + decltype(ic)::value;
-          sc[e / 16][mq][e % 16] = __builtin_fmaf(sc[e / 16][mq][e % 16], SL2, -msl[mq]);
+          sc[e / ACC_N][mq][e % ACC_N] = __builtin_fmaf(sc[e / ACC_N][mq][e % ACC_N], SL2, -msl[mq]);
         });
         if constexpr (t >= S_SLOTS && t - S_SLOTS < PVM) {
           constexpr int u = t - S_SLOTS;
@@ -695,7 +807,8 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
           constexpr int lo = (u * NM) / PVM, hi = ((u + 1) * NM) / PVM;
           static_for<hi - lo>([&](auto ic) {
             constexpr int i = lo + decltype(ic)::value;
-            mx[mq] = fmaxf(fmaxf(mx[mq], sn[i / 8][mq][(i % 8) * 2]), sn[i / 8][mq][(i % 8) * 2 + 1]);
+            mx[mq] = fmaxf(fmaxf(mx[mq], sn[2 * i / ACC_N][mq][2 * i % ACC_N]),
+                           sn[2 * i / ACC_N][mq][2 * i % ACC_N + 1]);
             pin(mx[mq]);
           });
         }
@@ -713,8 +826,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
         constexpr int pr = t / (2 * DK), r = t % (2 * DK), ks = r / 2, kt = 2 * pr + r % 2;
         static_for<MQ>([&](auto mqc) {
           constexpr int mq = decltype(mqc)::value;
-          sn[kt][mq] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
-              frag[t % 3], qf[mq][ks], ks == 0 ? zero : sn[kt][mq], 0, 0, 0);
+          sn[kt][mq] = DECA_MFMA(frag[t % 3], qf[mq][ks], ks == 0 ? zero : sn[kt][mq], 0, 0, 0);
         });
       } else {
         constexpr int u = t - S_SLOTS, kk = u / DT, dt = u % DT;
@@ -723,7 +835,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
           const half8 pfr = __builtin_shufflevector(
               __builtin_shufflevector(pf2[kk][mq][0], pf2[kk][mq][1], 0, 1, 2, 3),
               __builtin_shufflevector(pf2[kk][mq][2], pf2[kk][mq][3], 0, 1, 2, 3), 0, 1, 2, 3, 4, 5, 6, 7);
-          o_acc[dt][mq] = __builtin_amdgcn_mfma_f32_32x32x16_f16(frag[t % 3], pfr, o_acc[dt][mq], 0, 0, 0);
+          o_acc[dt][mq] = DECA_MFMA(frag[t % 3], pfr, o_acc[dt][mq], 0, 0, 0);
         });
       }
       valu(tc);
@@ -735,7 +847,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
   };
   half8 pf[KK][MQ];
   // tile j: softmax and second product; tile j+1: first product and row statistics
-  auto step = [&](auto cur_slot, floatx16 (&sc)[KT][MQ], floatx16 (&sn)[KT][MQ], int j) __attribute__((always_inline)) {
+  auto step = [&](auto cur_slot, acc_t (&sc)[KT][MQ], acc_t (&sn)[KT][MQ], int j) __attribute__((always_inline)) {
     constexpr int cur = decltype(cur_slot)::value;  // == j % 2
     wait_and_barrier();  // K_{j+1}, V_j landed; everyone is done with K_j and V_{j-1}
     if (j + 2 < nkv) issue_k(j + 2, cur);
@@ -745,7 +857,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
     rescale_o();
     fused(cur_slot, sc, sn);
   };
-  auto tail = [&](floatx16 (&sc)[KT][MQ], int j) __attribute__((always_inline)) {
+  auto tail = [&](acc_t (&sc)[KT][MQ], int j) __attribute__((always_inline)) {
     wait_and_barrier();
 #if DECA_CAUSAL
     // the diagonal tiles follow: V_{j+1} goes where V_{j-1} was (K_{j+1} is under way)
@@ -769,7 +881,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
   issue_v(0, 0);
   if (nd >= 2) {
     issue_k(1, 1);
-    floatx16 s_a[KT][MQ], s_b[KT][MQ];
+    acc_t s_a[KT][MQ], s_b[KT][MQ];
     wait_and_barrier();
     compute_s(s_a, 0);
     row_stats(s_a);
@@ -798,7 +910,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
   issue_k(0, 0);
   issue_v(0, 0);
   if (nkv > 1) issue_k(1, 1);
-  floatx16 s_a[KT][MQ], s_b[KT][MQ];
+  acc_t s_a[KT][MQ], s_b[KT][MQ];
   wait_and_barrier();
   compute_s(s_a, 0);
   row_stats(s_a);
@@ -865,7 +977,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
 #else
   for (int j = 0; j < nkv; ++j) {
     wait_and_barrier();
-    floatx16 s_acc[KT][MQ];
+    acc_t s_acc[KT][MQ];
     half8 pf[KK][MQ];
     compute_s(s_acc, 0);
     mask_s(s_acc, j);
@@ -897,18 +1009,19 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
   _Float16* o_lds = reinterpret_cast<_Float16*>(lds) + wave * WQ * EPI_LD;
 #pragma unroll
   for (int mq = 0; mq < MQ; ++mq) {
-    const float l = sum_halves(l_i[mq]);
+    const float l = sum_over_query(l_i[mq]);
     const float inv = 1.0f / l;
-    _Float16* o_row = EPI_LDS ? o_lds + (mq * 32 + l32) * EPI_LD + half * 4
-                              : o_base + (mq * 32 + l32) * D_ + half * 4;
+    // (16x16x32: o_acc[dt][mq][e]: q = mq*16 + lane%16, d = dt*16 + (lane/16)*4 + e)
+    _Float16* o_row = EPI_LDS ? o_lds + (mq * TQ + lq) * EPI_LD + lg * 4
+                              : o_base + (mq * TQ + lq) * D_ + lg * 4;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
+      for (int g = 0; g < ACC_N / 4; ++g) {
         half4 h;
 #pragma unroll
         for (int e = 0; e < 4; ++e) h[e] = static_cast<_Float16>(o_acc[dt][mq][g * 4 + e] * inv);
-        *reinterpret_cast<half4*>(o_row + dt * 32 + g * 8) = h;
+        *reinterpret_cast<half4*>(o_row + dt * TQ + g * 8) = h;
       }
   }
   if (EPI_LDS) {

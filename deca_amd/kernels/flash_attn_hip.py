@@ -44,6 +44,8 @@ class FAConfig:
     # before the softmax of tile j (two S^T accumulators).  2: as 1, and every matrix
     # instruction of an iteration carries a fixed share of its vector work.
     pipe: int = 0
+    # MFMA tile: 32 -> v_mfma_f32_32x32x16, 16 -> v_mfma_f32_16x16x32 (plain and slot loop)
+    mfma: int = 32
 
     @property
     def threads(self) -> int:
@@ -57,6 +59,7 @@ class FAConfig:
             f"Br={self.Br},Bc={self.Bc},warps={self.num_warps},stages={self.stages},"
             f"q_smem={int(self.q_in_smem)},swz={int(self.swizzle)}"
             + (f",pipe={int(self.pipe)}" if self.pipe else "")
+            + (f",mfma={self.mfma}" if self.mfma != 32 else "")
         )
 
 
@@ -107,16 +110,19 @@ def target_waves_per_simd(cfg: FAConfig, D: int) -> int:
     return max(1, min(by_regs, by_lds, 8))
 
 
-def slot_schedule_ok(Bc: int, D: int) -> bool:
+def slot_schedule_ok(Bc: int, D: int, mfma: int = 32) -> bool:
     """Whether the slot-interleaved loop (`pipe == 2`) can be scheduled: the S^T chains are
     issued in pairs, and the exponentials, spread over the matrix instructions at a fixed
     rate, must be packed before the O^T instruction that consumes them (the same check as
     `Sched::ok()` in the kernel)."""
-    kt, dk, kk, dt = Bc // 32, D // 16, Bc // 16, D // 32
+    if mfma == 16:
+        kt, dk, kk, dt, acc = Bc // 16, D // 32, Bc // 32, D // 16, 4
+    else:
+        kt, dk, kk, dt, acc = Bc // 32, D // 16, Bc // 16, D // 32, 16
     if Bc % 64 or kt % 2:
         return False
     s_slots, pv_slots = kt * dk, kk * dt
-    ns, ne = s_slots + pv_slots, kt * 16
+    ns, ne = s_slots + pv_slots, kt * acc
     ne_s, pve = ne * 5 // 8, pv_slots - dt - 2
     if pve < 1:
         return False
@@ -144,8 +150,10 @@ def check_config(cfg: FAConfig, S_q: int, S_kv: int, D: int) -> None:
     assert cfg.threads <= 1024
     assert cfg.stages in (1, 2)
     assert int(cfg.pipe) in (0, 1, 2)
+    assert cfg.mfma in (32, 16)
+    assert cfg.mfma == 32 or int(cfg.pipe) != 1, "the 16x16x32 form exists for the plain and the slot loop"
     assert not cfg.pipe or cfg.stages == 2
-    assert int(cfg.pipe) != 2 or slot_schedule_ok(cfg.Bc, D)
+    assert int(cfg.pipe) != 2 or slot_schedule_ok(cfg.Bc, D, cfg.mfma)
     assert not cfg.q_in_smem and cfg.swizzle
     assert smem_bytes(cfg, D) <= MAX_LDS
     assert est_regs_per_thread(cfg, D) <= 512
@@ -176,6 +184,8 @@ def make_flash_attn_fwd(
         "DECA_SCALE": repr(float(scale)), "DECA_PIPE": int(cfg.pipe),
         "DECA_MIN_WAVES": target_waves_per_simd(cfg, D), "DECA_LAZY_TAU": LAZY_MAX_TAU,
     }
+    if cfg.mfma == 16:
+        defines["DECA_MFMA16"] = 1
     return make_spec(
         TEMPLATE, defines, grid=((S_q // cfg.Br) * B * H, 1, 1), block=(cfg.threads, 1, 1), nargs=4,
         options=FAST_MATH_OPTIONS, meta={"cfg": str(cfg), "causal": causal},

@@ -64,3 +64,37 @@ def store(key: str, cfg, throughput: float, unit: str, path: str | None = None, 
         json.dump(table, f, indent=1, sort_keys=True)
         f.write("\n")
     os.replace(tmp, path)
+
+
+def parse_config(operator: str, text: str):
+    """The config object whose `str()` is `text` (the form the records and logs print),
+    e.g. "256x256x64,warp=128x64,stages=2,raster=0,epi_smem=1,mfma=16" for a GEMM."""
+    cls = _config_class(operator)
+    parts = [p for p in text.strip().split(",") if p]
+    fields = {}
+    if operator == "GEMM":
+        bm, bn, bk = (int(v) for v in parts.pop(0).split("x"))
+        fields.update(BM=bm, BN=bn, BK=bk)
+    pairs = dict(p.split("=", 1) for p in parts)
+    if operator == "GEMM":
+        wm, wn = (int(v) for v in pairs.pop("warp").split("x"))
+        fields.update(warp_m=wm, warp_n=wn, stages=int(pairs.pop("stages")),
+                      raster=int(pairs.pop("raster")), epi_smem=bool(int(pairs.pop("epi_smem"))),
+                      xcd=bool(int(pairs.pop("xcd", 1))), direct=bool(int(pairs.pop("direct", 1))),
+                      tail=bool(int(pairs.pop("tail", 0))), mfma=int(pairs.pop("mfma", 32)),
+                      early=int(pairs.pop("early", 0)))
+    elif operator in ("softmax", "rmsnorm"):
+        fields.update(threads_per_row=int(pairs.pop("tpr")), rows_per_block=int(pairs.pop("rpb")),
+                      vec=int(pairs.pop("vec")), mode=pairs.pop("mode"),
+                      unroll=int(pairs.pop("unroll", 1)), hint=bool(int(pairs.pop("hint", 0))))
+    else:
+        fields.update(Br=int(pairs.pop("Br")), Bc=int(pairs.pop("Bc")),
+                      num_warps=int(pairs.pop("warps")), stages=int(pairs.pop("stages")),
+                      q_in_smem=bool(int(pairs.pop("q_smem", 0))), swizzle=bool(int(pairs.pop("swz", 1))),
+                      pipe=int(pairs.pop("pipe", 0)), mfma=int(pairs.pop("mfma", 32)))
+    if pairs:
+        raise ValueError(f"unknown fields in {operator} config {text!r}: {sorted(pairs)}")
+    cfg = cls(**fields)
+    if str(cfg) != text.strip():
+        raise ValueError(f"{text!r} is not the canonical form {str(cfg)!r}")
+    return cfg

@@ -170,6 +170,20 @@ FA_CASES = [
     # key tiles wider than the query tiles
     (1, 2, 512, 512, 64, True, FAConfig(128, 128, 4, 2, pipe=2)),
     (1, 2, 1024, 1024, 64, True, FAConfig(64, 128, 2, 2, pipe=2)),
+    # 16x16x32 MFMA tiles (plain loop): full and causal, D = 64 / 128 / 192, one and two LDS
+    # stages, one and several query tiles per wave, S_q != S_kv
+    (1, 2, 256, 256, 128, False, FAConfig(128, 64, 4, 2, mfma=16)),
+    (1, 2, 512, 512, 128, True, FAConfig(256, 64, 8, 2, mfma=16)),
+    (2, 2, 512, 512, 64, True, FAConfig(128, 64, 4, 2, mfma=16)),
+    (1, 2, 256, 256, 64, False, FAConfig(256, 128, 4, 2, mfma=16)),
+    (1, 3, 128, 640, 128, False, FAConfig(64, 64, 2, 1, mfma=16)),
+    (1, 1, 128, 128, 128, True, FAConfig(32, 32, 1, 2, mfma=16)),
+    (1, 2, 256, 256, 192, True, FAConfig(128, 64, 4, 2, mfma=16)),
+    # ... in the slot loop: full, causal (odd and even numbers of unmasked tiles), D = 64
+    (1, 2, 512, 512, 128, False, FAConfig(256, 64, 8, 2, pipe=2, mfma=16)),
+    (1, 2, 512, 512, 128, True, FAConfig(256, 64, 8, 2, pipe=2, mfma=16)),
+    (1, 2, 512, 512, 64, True, FAConfig(128, 128, 4, 2, pipe=2, mfma=16)),
+    (2, 2, 512, 512, 64, False, FAConfig(128, 64, 4, 2, pipe=2, mfma=16)),
     # head dims that are multiples of 64 but no powers of two: full, causal, the three loops
     (1, 2, 256, 256, 192, False, FAConfig(128, 64, 4, 2)),
     (1, 2, 256, 256, 192, True, FAConfig(128, 64, 4, 2)),

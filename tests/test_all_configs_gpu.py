@@ -33,6 +33,17 @@ def _build_all(specs):
         return list(pool.map(cached_build, specs))
 
 
+def _launch(what, kern, *args):
+    """One launch, named on stdout before it starts; a HIP error ends the whole session (the
+    device is not to be used after a fault), a wrong result is only collected by the caller."""
+    print(f"launch {what}", flush=True)
+    try:
+        kern(*args)
+        torch.cuda.synchronize()
+    except RuntimeError as err:
+        pytest.exit(f"HIP error in {what}: {err}", returncode=3)
+
+
 def _arch():
     from deca_amd.arch.MI355X import MI355X
 
@@ -54,8 +65,7 @@ def test_every_flash_attn_config(B, H, S, D, causal):
     wrong = []
     for cfg, spec, path in zip(configs, specs, paths):
         o = torch.full_like(q, float("nan"))
-        load_kernel(spec, path)(q, k, v, o)
-        torch.cuda.synchronize()
+        _launch(f"fa B{B} H{H} S{S} D{D} causal={causal} {cfg}", load_kernel(spec, path), q, k, v, o)
         err = (o.float() - ref).abs().max().item()
         if not err <= 2e-3:
             wrong.append((str(cfg), err))
@@ -78,8 +88,7 @@ def test_every_gemm_config(M, N, K):
     wrong = []
     for cfg, spec, path in zip(configs, specs, paths):
         c = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
-        load_kernel(spec, path)(a, b, c)
-        torch.cuda.synchronize()
+        _launch(f"gemm {M}x{N}x{K} {cfg}", load_kernel(spec, path), a, b, c)
         err = (c.float() - ref).abs().max().item() / scale
         if not err <= 1e-2:
             wrong.append((str(cfg), err))
@@ -107,8 +116,7 @@ def test_every_rowwise_config(op, M, N, dtype):
     wrong = []
     for cfg, spec, path in zip(configs, specs, paths):
         y = torch.full_like(inputs[0], float("nan"))
-        load_kernel(spec, path)(*inputs, y)
-        torch.cuda.synchronize()
+        _launch(f"{op} {dtype} {M}x{N} {cfg}", load_kernel(spec, path), *inputs, y)
         err = ((y.float() - ref).abs() / ref.abs().clamp(min=1.0)).max().item()
         if not err <= tol:
             wrong.append((str(cfg), err))

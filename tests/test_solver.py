@@ -140,9 +140,9 @@ def test_flash_attn_configs_are_valid(D, S):
         fa.check_config(cfg, S, S, D)
         assert (S // cfg.Br) * B * H >= ARCH.sm_nums
     want = set()
-    for br, bc, nw, st, pipe in itertools.product((32, 64, 128, 256), (32, 64, 128), (1, 2, 4, 8),
-                                                   (1, 2), (0, 1, 2)):
-        cfg = fa.FAConfig(br, bc, nw, st, pipe=pipe)
+    for br, bc, nw, st, pipe, mfma in itertools.product(
+            (32, 64, 128, 256), (32, 64, 128), (1, 2, 4, 8), (1, 2), (0, 1, 2), (32, 16)):
+        cfg = fa.FAConfig(br, bc, nw, st, pipe=pipe, mfma=mfma)
         try:
             fa.check_config(cfg, S, S, D)
         except AssertionError:

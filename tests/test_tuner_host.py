@@ -245,3 +245,26 @@ def test_rotating_sets_and_cycle():
     for _ in range(6):
         call()
     assert seen[:4] == [s[-1].data_ptr() for s in sets] and seen[4:] == seen[:2]
+
+
+def test_config_strings_parse_back():
+    """Every config's printed form (what records, logs and bench.py --kernel-config use)
+    parses back into the same object."""
+    from deca_amd import tuned
+    from deca_amd.kernels.flash_attn_hip import FAConfig
+    from deca_amd.kernels.gemm_hip import GemmConfig
+    from deca_amd.kernels.rowwise_hip import RowConfig
+
+    cases = [
+        ("GEMM", GemmConfig(256, 256, 64, 128, 64, 2, 0, True, True, True)),
+        ("GEMM", GemmConfig(128, 128, 32, 64, 32, 5, 4, False, False, True, True, 16, 2)),
+        ("GEMM", GemmConfig(256, 128, 64, 128, 64, 1, 1, True, False, False)),
+        ("softmax", RowConfig(256, 2, 8, "reg", 1, True)),
+        ("rmsnorm", RowConfig(1024, 1, 4, "twopass", 4)),
+        ("flash_attn", FAConfig(256, 64, 8, 2, pipe=2)),
+        ("flash_attn", FAConfig(128, 128, 4, 1)),
+    ]
+    for op, cfg in cases:
+        assert tuned.parse_config(op, str(cfg)) == cfg
+    with pytest.raises(ValueError):
+        tuned.parse_config("GEMM", "256x256x64,warp=128x64,stages=2,raster=0,epi_smem=1,bogus=1")
