@@ -10,6 +10,9 @@ arch files as comments (arch/H20.py:35-60); here they can be taken again:
 - HBM: a 16-byte-per-lane copy, a read-only and a write-only stream of 128 MiB
   buffers, rotating over 8 buffer pairs (2 GiB, several times the 256 MiB Infinity
   Cache) so that every launch streams from memory.
+- LDS and the L2 -> LDS path: per workgroup of 8 waves (one workgroup per CU), some waves
+  stream conflict-free ds_read_b128, others direct global->LDS loads from an L2-resident
+  region; alone and together, which shows what the two share.
 - Matrix pipe: register-only loops of v_mfma_f32_32x32x16_f16 and
   v_mfma_f32_16x16x32_f16 (no memory traffic) on N(0,1) and on all-zero operands:
   with real data the board's power limit, not its 2.4 GHz clock, sets the rate.
@@ -46,6 +49,15 @@ def mfma_spec(mode: int, nacc: int, blocks: int):
                                 "DECA_NACC": nacc}, (blocks, 1, 1), (256, 1, 1), 2, options=[])
 
 
+LDS_ITERS = 4000
+LDS_MIXES = [(8, 0), (4, 0), (0, 4), (0, 2), (4, 4), (6, 2)]  # (reading waves, loading waves)
+
+
+def lds_spec(readers: int, loaders: int):
+    return make_spec(TEMPLATE, {"DECA_CEILING": 5, "DECA_READERS": readers, "DECA_LOADERS": loaders,
+                                "DECA_ITERS": LDS_ITERS}, (256, 1, 1), (512, 1, 1), 2, options=[])
+
+
 STREAM_VARIANTS = [(t, u, nt, w) for t, u, nt, w in itertools.product(
     (256, 512, 1024), (1, 2, 4), (0, 1), (0, 2048))]
 MFMA_VARIANTS = [(3, 8, 1024), (3, 8, 2048), (4, 16, 1024), (4, 16, 2048)]
@@ -53,7 +65,7 @@ MFMA_VARIANTS = [(3, 8, 1024), (3, 8, 2048), (4, 16, 1024), (4, 16, 2048)]
 
 def all_specs():
     specs = [stream_spec(m, *v) for m in (0, 1, 2) for v in STREAM_VARIANTS]
-    return specs + [mfma_spec(*v) for v in MFMA_VARIANTS]
+    return specs + [mfma_spec(*v) for v in MFMA_VARIANTS] + [lds_spec(*m) for m in LDS_MIXES]
 
 
 def build():
@@ -89,6 +101,27 @@ def measure_streams(out=sys.stdout):
               f"{threads} lanes, {unroll} in flight, {'non-temporal' if nt else 'plain'}, "
               f"{'grid-stride over ' + str(wgs) + ' workgroups' if wgs else 'one pass per lane'})",
               file=out, flush=True)
+
+
+def measure_lds(out=sys.stdout):
+    """Bytes per nominal 2.4 GHz clock and CU (these loops draw little power: the shader
+    clock stays at its maximum)."""
+    import torch
+
+    from deca_amd.driver.driver import load_kernel
+
+    src = torch.zeros(65 * 65536, dtype=torch.uint8, device="cuda")
+    res = torch.empty(256 * 512, device="cuda")
+    for readers, loaders in LDS_MIXES:
+        spec = lds_spec(readers, loaders)
+        kern = load_kernel(spec, cached_build(spec))
+        kern.time([(src, res)], 1)
+        t = min(kern.time([(src, res)], 3) for _ in range(3))
+        clocks = t * 2.4e9
+        per_wave = LDS_ITERS * 8 * 1024
+        print(f"LDS: {readers} waves ds_read_b128 + {loaders} waves global->LDS per CU: {t * 1e3:.3f} ms; "
+              f"had each stream run all of it: reads {readers * per_wave / clocks:5.1f} B/clk/CU, "
+              f"loads {loaders * per_wave / clocks:5.1f} B/clk/CU", file=out, flush=True)
 
 
 def measure_mfma(out=sys.stdout):
@@ -164,6 +197,7 @@ def main(argv=None):
     if args.build:
         return
     measure_streams()
+    measure_lds()
     measure_mfma()
     if args.sclk:
         measure_sclk()

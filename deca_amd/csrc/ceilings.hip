@@ -8,17 +8,58 @@
 //                2  write only  16-byte stores of a lane-dependent constant
 //                3  matrix      register-only loop of v_mfma_f32_32x32x16_f16
 //                4  matrix      register-only loop of v_mfma_f32_16x16x32_f16
+//                5  LDS / L2    8 waves per workgroup: DECA_READERS of them stream conflict-free
+//                               ds_read_b128, DECA_LOADERS stream direct global->LDS loads
+//                               (global_load_lds_dwordx4) from a 4 MiB, L2-resident region,
+//                               DECA_ITERS trips of 8 KiB per wave each
 //   DECA_THREADS    lanes per workgroup
 //   DECA_CHUNKS     (0..2) 16-byte chunks of the buffer; DECA_UNROLL accesses in flight per lane;
 //                   DECA_NT 1: non-temporal loads / stores
 //   DECA_ITERS      (3, 4) loop trips, DECA_NACC independent accumulator tiles per wave
 #include <hip/hip_runtime.h>
 
+#pragma clang diagnostic ignored "-Winline-asm"  // M0 is set and declared clobbered on purpose
+
 typedef float f4 __attribute__((ext_vector_type(4)));
 typedef float f16v __attribute__((ext_vector_type(16)));
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 
-#if DECA_CEILING <= 2
+#if DECA_CEILING == 5
+extern "C" __global__ void __launch_bounds__(512)
+deca_main(const unsigned char* __restrict__ in, float* __restrict__ out) {
+  __shared__ __attribute__((aligned(16))) unsigned char lds[128 * 1024];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  for (int i = threadIdx.x; i < 32768; i += 512) reinterpret_cast<float*>(lds)[i] = static_cast<float>(i);
+  __syncthreads();
+  f4 acc = {0.f, 0.f, 0.f, 0.f};
+  if (wave < DECA_READERS) {
+    const unsigned char* p = lds + wave * 8192 + lane * 16;
+    for (int it = 0; it < DECA_ITERS; ++it) {
+#pragma unroll
+      for (int u = 0; u < 8; ++u) acc += *reinterpret_cast<const f4*>(p + u * 1024);
+    }
+  } else if (wave < DECA_READERS + DECA_LOADERS) {
+    // lane L's 16 bytes land at (wave-uniform LDS base in M0) + 16 L
+    const unsigned dst = static_cast<unsigned>(reinterpret_cast<size_t>(
+        (__attribute__((address_space(3))) void*)(lds + 65536 + (wave - DECA_READERS) * 8192)));
+    const unsigned voff = lane * 16;
+    const unsigned char* src = in + (blockIdx.x & 63) * 65536 + (wave - DECA_READERS) * 8192;
+    for (int it = 0; it < DECA_ITERS; ++it) {
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                     :
+                     : "v"(voff), "s"(src + u * 1024), "s"(dst + u * 1024)
+                     : "memory", "m0");
+      __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8): one trip stays in flight
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+  }
+  __syncthreads();
+  out[blockIdx.x * 512 + threadIdx.x] = acc.x + acc.y + acc.z + acc.w + lds[threadIdx.x * 4 + 65536];
+}
+#elif DECA_CEILING <= 2
 extern "C" __global__ void __launch_bounds__(DECA_THREADS)
 deca_main(const f4* __restrict__ in, f4* __restrict__ out) {
   const long tid = static_cast<long>(blockIdx.x) * DECA_THREADS + threadIdx.x;
