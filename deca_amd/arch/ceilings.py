@@ -13,6 +13,8 @@ arch files as comments (arch/H20.py:35-60); here they can be taken again:
 - LDS and the L2 -> LDS path: per workgroup of 8 waves (one workgroup per CU), some waves
   stream conflict-free ds_read_b128, others direct global->LDS loads from an L2-resident
   region; alone and together, which shows what the two share.
+- Vector ALU: register-only loops of the instructions the softmax of FlashAttention is made
+  of, and of an MFMA followed by such work in the same wave (what one wave overlaps by itself).
 - Matrix pipe: register-only loops of v_mfma_f32_32x32x16_f16 and
   v_mfma_f32_16x16x32_f16 (no memory traffic) on N(0,1) and on all-zero operands:
   with real data the board's power limit, not its 2.4 GHz clock, sets the rate.
@@ -58,6 +60,29 @@ def lds_spec(readers: int, loaders: int):
                                 "DECA_ITERS": LDS_ITERS}, (256, 1, 1), (512, 1, 1), 2, options=[])
 
 
+VALU_ITERS = 4096
+VALU_OPS = {0: "16 v_fma_f32", 1: "16 v_exp_f32", 2: "16 v_cvt_pk_f16_f32", 3: "16 v_max3_f32",
+            4: "4 x (MFMA 32x32x16 + 2 v_exp_f32)", 5: "4 x (MFMA 32x32x16 + 8 v_fma_f32)",
+            6: "4 x MFMA 32x32x16",
+            7: "4 x (MFMA 32x32x16 + 2 v_fma_f32 + v_exp_f32 + v_cvt_pk_f16_f32 + v_max3_f32)",
+            8: "4 x (MFMA 32x32x16 + 2 x (2 v_fma_f32 + v_exp_f32 + v_cvt_pk_f16_f32 + v_max3_f32))",
+            9: "4 x (MFMA 32x32x16 + 2 x (2 v_fma_f32 + v_exp_f32 + v_cvt_pk_f16_f32 + v_max3_f32) "
+               "+ 2 v_accvgpr_read_b32)",
+            10: "16 dependent v_fma_f32", 11: "16 dependent v_exp_f32", 12: "16 dependent v_max3_f32",
+            13: "16 x (v_exp_f32, dependent v_add_f32)"}
+VALU_CHAIN_OPS = (0, 1, 10, 11, 12, 13)  # these also run with one and two waves per SIMD
+
+
+VALU_RUNS = [(op, 0) for op in VALU_OPS if op != 9 and op < 10] + [(4, 1), (5, 1), (6, 1), (7, 1), (8, 1), (9, 1)]
+
+
+def valu_spec(op: int, agpr: int = 0, waves_per_simd: int = 8):
+    blocks = 256 * waves_per_simd
+    return make_spec(TEMPLATE, {"DECA_CEILING": 6, "DECA_OP": op, "DECA_ITERS": VALU_ITERS,
+                                "DECA_ACC_AGPR": agpr},
+                     (blocks, 1, 1), (256, 1, 1), 2, options=[])
+
+
 STREAM_VARIANTS = [(t, u, nt, w) for t, u, nt, w in itertools.product(
     (256, 512, 1024), (1, 2, 4), (0, 1), (0, 2048))]
 MFMA_VARIANTS = [(3, 8, 1024), (3, 8, 2048), (4, 16, 1024), (4, 16, 2048)]
@@ -65,7 +90,9 @@ MFMA_VARIANTS = [(3, 8, 1024), (3, 8, 2048), (4, 16, 1024), (4, 16, 2048)]
 
 def all_specs():
     specs = [stream_spec(m, *v) for m in (0, 1, 2) for v in STREAM_VARIANTS]
-    return specs + [mfma_spec(*v) for v in MFMA_VARIANTS] + [lds_spec(*m) for m in LDS_MIXES]
+    return (specs + [mfma_spec(*v) for v in MFMA_VARIANTS] + [lds_spec(*m) for m in LDS_MIXES]
+            + [valu_spec(op, agpr) for op, agpr in VALU_RUNS]
+            + [valu_spec(op, 0, w) for op in VALU_CHAIN_OPS for w in (1, 2)])
 
 
 def build():
@@ -124,6 +151,28 @@ def measure_lds(out=sys.stdout):
               f"loads {loaders * per_wave / clocks:5.1f} B/clk/CU", file=out, flush=True)
 
 
+def measure_valu(out=sys.stdout):
+    """Clocks per trip and SIMD at the nominal 2.4 GHz: 2048 workgroups of 4 waves are 8 waves
+    per SIMD over the 256 CUs, all resident at once."""
+    import torch
+
+    from deca_amd.driver.driver import load_kernel
+
+    x = torch.rand(8192, device="cuda")
+    x[4096:] = 0  # the MFMA operands: zeros draw no power, the clock stays at its maximum
+    res = torch.empty(2048 * 256, device="cuda")
+    runs = [(op, agpr, 8) for op, agpr in VALU_RUNS] + [(op, 0, w) for op in VALU_CHAIN_OPS for w in (1, 2)]
+    for op, agpr, waves in runs:
+        what = VALU_OPS[op] + (", accumulators in AGPRs" if agpr else "")
+        spec = valu_spec(op, agpr, waves)
+        kern = load_kernel(spec, cached_build(spec))
+        kern.time([(x, res)], 1)
+        t = min(kern.time([(x, res)], 3) for _ in range(3))
+        clocks = t * 2.4e9 / VALU_ITERS / waves
+        print(f"VALU: {what} per trip, {waves} waves per SIMD: {t * 1e3:.3f} ms, {clocks:6.1f} clocks per trip "
+              f"and wave", file=out, flush=True)
+
+
 def measure_mfma(out=sys.stdout):
     import torch
 
@@ -144,48 +193,81 @@ def measure_mfma(out=sys.stdout):
                   f"{flops / t / 1e12:6.0f} TFLOP/s ({t * 1e3:.3f} ms)", file=out, flush=True)
 
 
-def _sclk():
+def _board_state():
+    """Shader clock, socket power and power cap as rocm-smi reports them, on one line."""
     try:
-        text = subprocess.run(["rocm-smi", "--showclocks"], capture_output=True, text=True,
-                              timeout=20).stdout
+        text = subprocess.run(["rocm-smi", "--showclocks", "--showpower", "--showmaxpower"],
+                              capture_output=True, text=True, timeout=20).stdout
     except (OSError, subprocess.SubprocessError) as err:
         return f"rocm-smi failed: {err}"
-    return " | ".join(line.strip() for line in text.splitlines() if "sclk" in line)
+    keep = [line.split(":", 1)[1].strip() for line in text.splitlines()
+            if "sclk" in line or "Power (W)" in line]
+    try:  # the socket power comes from amd-smi where rocm-smi does not print it
+        text = subprocess.run(["amd-smi", "metric", "-p"], capture_output=True, text=True, timeout=20).stdout
+        keep += [line.strip() for line in text.splitlines() if "SOCKET_POWER" in line]
+    except (OSError, subprocess.SubprocessError):
+        pass
+    return " | ".join(keep)
+
+
+def _sample_while(launch, label, out, seconds=3):
+    """Prints the board state once a second while `launch()` (a batch of asynchronous
+    launches) repeats on a worker thread."""
+    import torch
+
+    stop = threading.Event()
+
+    def work():
+        while not stop.is_set():
+            launch()
+            torch.cuda.synchronize()
+
+    worker = threading.Thread(target=work)
+    worker.start()
+    for _ in range(seconds):
+        time.sleep(1.0)
+        print(f"{label}: {_board_state()}", file=out, flush=True)
+    stop.set()
+    worker.join()
 
 
 def measure_sclk(out=sys.stdout):
-    """Shader clock reported by rocm-smi while the tuned 8192^3 GEMM loops."""
+    """Shader clock and socket power reported by rocm-smi while the tuned 8192^3 GEMM, the
+    tuned FlashAttention kernels and the register-only MFMA loop repeat."""
     import torch
 
     from deca_amd import tuned
+    from deca_amd.driver.driver import load_kernel
+    from deca_amd.kernels.attn_bench import attn_flops, make_qkv
+    from deca_amd.kernels.flash_attn_hip import build_flash_attn, make_flash_attn_fwd
     from deca_amd.kernels.gemm_hip import build_gemm_tc, make_gemm_tc
 
     n = 8192
     cfg = tuned.lookup(tuned.make_key("GEMM", (n, n, n), "float16", "gfx950", False))
     kern = build_gemm_tc(make_gemm_tc(n, n, n, cfg))
-    print(f"idle: {_sclk()}", file=out, flush=True)
+    print(f"idle: {_board_state()}", file=out, flush=True)
     makers = {"U(-1,1)": lambda: (2 * torch.rand(n, n, device="cuda") - 1).half(),
               "zeros": lambda: torch.zeros(n, n, device="cuda", dtype=torch.float16)}
     for name, make in makers.items():
         a, b = make(), make()
         c = torch.empty(n, n, device="cuda", dtype=torch.float16)
-        stop = threading.Event()
-
-        def work():
-            while not stop.is_set():
-                for _ in range(50):
-                    kern(a, b, c)
-                torch.cuda.synchronize()
-
-        worker = threading.Thread(target=work)
-        worker.start()
-        for _ in range(3):
-            time.sleep(1.0)
-            print(f"GEMM {n}^3 [{cfg}] on {name}: {_sclk()}", file=out, flush=True)
-        stop.set()
-        worker.join()
+        _sample_while(lambda: [kern(a, b, c) for _ in range(50)], f"GEMM {n}^3 [{cfg}] on {name}", out)
         t = kern.time([(a, b, c)], 20)
         print(f"  -> {2 * n**3 / t / 1e12:.0f} TFLOP/s", file=out, flush=True)
+    for d in (128, 64):
+        shape = (4, 16, 4096, 4096, d)
+        fcfg = tuned.lookup(tuned.make_key("flash_attn", shape, "float16", "gfx950", False))
+        fa = build_flash_attn(make_flash_attn_fwd(*shape, fcfg, None, False))
+        q, k, v = make_qkv(*shape)
+        o = torch.empty_like(q)
+        _sample_while(lambda: [fa(q, k, v, o) for _ in range(50)], f"FlashAttention D{d} [{fcfg}] on N(0,1)", out)
+        t = fa.time([(q, k, v, o)], 20)
+        print(f"  -> {attn_flops(*shape, False) / t / 1e12:.0f} TFLOP/s", file=out, flush=True)
+    spec = mfma_spec(3, 8, 2048)
+    loop = load_kernel(spec, cached_build(spec))
+    x = torch.randn(4096 * 8, device="cuda").half()
+    res = torch.empty(2048 * 256, device="cuda")
+    _sample_while(lambda: [loop(x, res) for _ in range(10)], "MFMA 32x32x16 register-only loop on N(0,1)", out)
 
 
 def main(argv=None):
@@ -198,6 +280,7 @@ def main(argv=None):
         return
     measure_streams()
     measure_lds()
+    measure_valu()
     measure_mfma()
     if args.sclk:
         measure_sclk()

@@ -12,6 +12,8 @@
 //                               ds_read_b128, DECA_LOADERS stream direct global->LDS loads
 //                               (global_load_lds_dwordx4) from a 4 MiB, L2-resident region,
 //                               DECA_ITERS trips of 8 KiB per wave each
+//                6  vector ALU  register-only loops of one instruction (DECA_OP), 16 independent
+//                               chains per lane, and of an MFMA with vector work behind it
 //   DECA_THREADS    lanes per workgroup
 //   DECA_CHUNKS     (0..2) 16-byte chunks of the buffer; DECA_UNROLL accesses in flight per lane;
 //                   DECA_NT 1: non-temporal loads / stores
@@ -24,7 +26,108 @@ typedef float f4 __attribute__((ext_vector_type(4)));
 typedef float f16v __attribute__((ext_vector_type(16)));
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 
-#if DECA_CEILING == 5
+#if DECA_CEILING == 6
+// DECA_OP 0 v_fma_f32, 1 v_exp_f32, 2 v_cvt_pk_f16_f32 (packs two results), 3 v_max3_f32,
+// 4 one 32x32x16 MFMA (zero operands) followed by two v_exp_f32 in the same wave, 5 the same
+// with eight v_fma_f32, 6 the MFMAs alone, 7 an MFMA followed by the softmax mix of a
+// FlashAttention tile (2 fma, 1 exp, 1 cvt_pk, 1 max3), 8 that mix twice per MFMA (head
+// dim 64), 9 the same plus two reads of accumulation registers,
+// 10-12 sixteen v_fma_f32 / v_exp_f32 / v_max3_f32 that each consume the one before, 13 sixteen
+// v_exp_f32 each followed by a v_add_f32 that consumes it; DECA_ACC_AGPR 1 keeps the MFMA accumulators in
+// the accumulation half of the register file
+extern "C" __global__ void __launch_bounds__(256)
+deca_main(const float* __restrict__ in, float* __restrict__ out) {
+  float x[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) x[i] = in[(threadIdx.x + i * 256) % 4096];
+  const float c0 = in[threadIdx.x], c1 = in[threadIdx.x + 1];
+#if DECA_OP >= 4
+  half8 a, b;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    a[i] = static_cast<_Float16>(in[4096 + (threadIdx.x + i) % 4096]);  // the host keeps this half zero:
+    b[i] = static_cast<_Float16>(in[4096 + (threadIdx.x * 3 + i) % 4096]);  // no power limit on the MFMAs
+  }
+  f16v acc[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[i][e] = 0.f;
+#endif
+  for (int it = 0; it < DECA_ITERS; ++it) {
+#if DECA_OP >= 10
+    // one dependent chain: what a wave waits between an instruction and its consumer
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+#if DECA_OP == 10
+      asm volatile("v_fma_f32 %0, %0, %1, %2" : "+v"(x[0]) : "v"(c0), "v"(c1));
+#elif DECA_OP == 11
+      asm volatile("v_exp_f32 %0, %0" : "+v"(x[0]));
+#elif DECA_OP == 12
+      asm volatile("v_max3_f32 %0, %0, %1, %2" : "+v"(x[0]) : "v"(c0), "v"(c1));
+#else
+      asm volatile("v_exp_f32 %0, %0\n\tv_add_f32 %1, %1, %0" : "+v"(x[i]), "+v"(x[(i + 1) % 16]));
+#endif
+    }
+#elif DECA_OP < 4
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+#if DECA_OP == 0
+      asm volatile("v_fma_f32 %0, %0, %1, %2" : "+v"(x[i]) : "v"(c0), "v"(c1));
+#elif DECA_OP == 1
+      asm volatile("v_exp_f32 %0, %0" : "+v"(x[i]));
+#elif DECA_OP == 2
+      asm volatile("v_cvt_pk_f16_f32 %0, %0, %1" : "+v"(x[i]) : "v"(c0));
+#else
+      asm volatile("v_max3_f32 %0, %0, %1, %2" : "+v"(x[i]) : "v"(c0), "v"(c1));
+#endif
+    }
+#else
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+#if DECA_ACC_AGPR
+      asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(acc[i]) : "v"(a), "v"(b));
+#else
+      acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc[i], 0, 0, 0);
+#endif
+#if DECA_OP == 4
+      asm volatile("v_exp_f32 %0, %0\n\tv_exp_f32 %1, %1" : "+v"(x[2 * i]), "+v"(x[2 * i + 1]));
+#elif DECA_OP == 7
+      asm volatile("v_fma_f32 %0, %0, %4, %5\n\tv_exp_f32 %1, %1\n\tv_fma_f32 %2, %2, %4, %5\n\t"
+                   "v_cvt_pk_f16_f32 %3, %3, %4\n\tv_max3_f32 %0, %0, %4, %5"
+                   : "+v"(x[4 * i]), "+v"(x[4 * i + 1]), "+v"(x[4 * i + 2]), "+v"(x[4 * i + 3])
+                   : "v"(c0), "v"(c1));
+#elif DECA_OP == 8 || DECA_OP == 9
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        asm volatile("v_fma_f32 %0, %0, %4, %5\n\tv_exp_f32 %1, %1\n\tv_fma_f32 %2, %2, %4, %5\n\t"
+                     "v_cvt_pk_f16_f32 %3, %3, %4\n\tv_max3_f32 %0, %0, %4, %5"
+                     : "+v"(x[4 * i]), "+v"(x[4 * i + 1]), "+v"(x[4 * i + 2]), "+v"(x[4 * i + 3])
+                     : "v"(c0), "v"(c1));
+#if DECA_OP == 9 && DECA_ACC_AGPR
+      asm volatile("v_accvgpr_read_b32 %0, %2\n\tv_accvgpr_read_b32 %1, %3"
+                   : "=v"(x[(4 * i + 5) % 16]), "=v"(x[(4 * i + 6) % 16]) : "a"(acc[(i + 2) % 4][0]), "a"(acc[(i + 2) % 4][1]));
+#endif
+#elif DECA_OP == 5
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        asm volatile("v_fma_f32 %0, %0, %1, %2" : "+v"(x[(4 * i + j) % 16]) : "v"(c0), "v"(c1));
+#endif
+    }
+#endif
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) s += x[i];
+#if DECA_OP >= 4
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) s += acc[i][e];
+#endif
+  out[blockIdx.x * 256 + threadIdx.x] = s;
+}
+#elif DECA_CEILING == 5
 extern "C" __global__ void __launch_bounds__(512)
 deca_main(const unsigned char* __restrict__ in, float* __restrict__ out) {
   __shared__ __attribute__((aligned(16))) unsigned char lds[128 * 1024];
