@@ -300,6 +300,8 @@ def _gemm_constraints(arch, M: int, N: int, K: int, type_size: int):
             o.implies(o.eq(mfma, c(16)), o.eq(direct, c(1))),
             o.implies(o.all_of(o.eq(mfma, c(16)), o.eq(bk, c(32))),
                       o.eq(o.urem(o.udiv(k_, bk), c(2)), c(0))),
+            # at most 32 accumulator tiles of 16 x 16 per wave: 128 x 128 wave tiles spill
+            o.implies(o.eq(mfma, c(16)), o.ule(o.udiv(wm, c(16)) * o.udiv(wn, c(16)), c(32))),
             # 1 to 16 waves per workgroup
             o.uge(threads, c(wave)), o.ule(threads, c(arch.max_threads_per_block)),
             # cooperative 16-byte loads (and epilogue stores) evenly cover the tiles

@@ -320,6 +320,12 @@ def fa_score(cfg, arch, shape, causal: bool = False) -> float:
     # chain for nothing in return (measured 2-8 % behind the plain loop of the same tile)
     if int(cfg.pipe) == 1:
         pipe *= 0.90
+    # 16x16x32 tiles: twice the matrix instructions and LDS fragment reads per FLOP for
+    # the same vector work.  Measured 0-3 % behind the 32x32x16 twin on full shapes (ranked
+    # just behind it there, so that the twins do not fill the measured top-N) and 2-8 %
+    # ahead of it under the causal mask at D = 128 (the twins stay tied there).
+    if getattr(cfg, "mfma", 32) == 16 and not causal:
+        pipe *= 0.97
     sync = 1.0 / (1.0 + getattr(arch, "fa_cta_sync_penalty", 0.0) * cfg.num_warps / 4 / wgs)
     # longer KV steps amortise the per-step max / barrier; the slot loop has the row
     # statistics inside the matrix work and pays a little less of it

@@ -1,20 +1,20 @@
 // 16-bit x 16-bit -> fp32-accumulate GEMM, C[M,N] = A[M,K] * B[K,N], all row-major
 // float16 (or bfloat16 with DECA_BF16), for gfx950 (MFMA v_mfma_f32_32x32x16_f16 /
-// _bf16).
+// _bf16, or the 16x16x32 forms with DECA_MFMA16).
 //
 // One code object per (shape, GemmConfig); every DECA_* macro is a compile-time
 // constant supplied by kernels/gemm_hip.py, as the reference bakes shape and
 // config into each generated kernel (src/kernels/gemm_tir.py:123-156).
 //
 //   DECA_M/N/K    problem size          DECA_BM/BN/BK  workgroup tile
-//   DECA_WM/WN    wave tile             DECA_STAGES    LDS ring depth (1 or 2)
+//   DECA_WM/WN    wave tile             DECA_STAGES    LDS ring depth (see DECA_DIRECT)
 //   DECA_RASTER   workgroup rows per rasterisation group; 0: an 8 x 4 sub-block of
 //                 tiles per XCD, 8 neighbouring sub-blocks in flight
 //   DECA_EPI_LDS  1: stage C through LDS for 16-byte stores
 //   DECA_XCD      1: remap workgroup ids so that each of the 8 XCDs (private L2)
 //                 owns a contiguous slab of tiles
 //   DECA_DIRECT   1: global -> LDS loads that bypass the VGPRs, ring of
-//                 DECA_STAGES (2..4) tiles; 0: loads staged through VGPRs one
+//                 DECA_STAGES (2..5) tiles; 0: loads staged through VGPRs one
 //                 tile ahead, ring of 1 or 2 tiles
 //   DECA_TAIL     R > 0: the last R tiles (the partial last wave of workgroups)
 //                 are computed as 4 R quarter tiles of BM/2 x BN/2, by

@@ -21,8 +21,9 @@
 // Lane t of a row owns the VEC-element chunks (c * TPR + t) * VEC, so one wave
 // touches 64 * VEC * 2 contiguous bytes per access (1 KiB at VEC = 8).
 // Reductions: DPP butterflies inside a wave (quad_perm, row_half_mirror,
-// row_mirror), ds_swizzle / ds_bpermute across the 16- and 32-lane halves,
-// then an LDS exchange between the waves of a row.  All math is fp32.
+// row_mirror), v_permlane16_swap / v_permlane32_swap across the 16- and 32-lane
+// halves (register exchanges, no LDS pipe), then an LDS exchange between the waves
+// of a row.  All math is fp32.
 //
 // Numerics follow src/kernels/rowwise_tir.py:278-389:
 //   softmax: m2 = max(x) * log2e; y = exp2(x * log2e - m2) * (1 / sum)

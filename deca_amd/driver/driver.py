@@ -186,6 +186,10 @@ def get_driver() -> HipDriver:
     return _driver
 
 
+class KernelRejected(RuntimeError):
+    """A code object that loads but must not be launched (see LoadedKernel)."""
+
+
 class LoadedKernel:
     """A code object loaded on the device plus its launch geometry.
 
@@ -203,6 +207,19 @@ class LoadedKernel:
         self.fn = self.drv.get_function(self.mod, spec.symbol)
         if spec.lds_bytes > 64 * 1024:
             self.drv.set_max_dynamic_lds(self.fn, spec.lds_bytes)
+        # A kernel whose loop waits for "all but the newest n" of its global->LDS loads
+        # (s_waitcnt vmcnt(n), n > 0) counts on those loads being the loop's only vector
+        # memory traffic.  Register spills put scratch stores into the same counter, and
+        # stores retire out of order with respect to loads: the wait may then pass with a
+        # tile still in flight.  Such a code object is refused instead of launched.
+        meta = dict(spec.meta)
+        if meta.get("no_scratch"):
+            scratch = self.info()["scratch_bytes"]
+            if scratch > 0:
+                self.close()
+                raise KernelRejected(
+                    f"{spec.template} [{meta.get('cfg', '')}] spills {scratch} bytes per lane to "
+                    "scratch memory; its partial vmcnt waits are only valid without spills")
 
     def info(self) -> dict:
         return self.drv.function_info(self.fn)

@@ -170,6 +170,8 @@ def kernel_resources(spec: KernelSpec, arch: str | None = None) -> dict:
         with open(asm) as f:
             for line in f:
                 s = line.strip()
+                if s.startswith("- "):  # the first key of a kernel's metadata entry
+                    s = s[2:].lstrip()
                 for k, name in keys.items():
                     if s.startswith(k):
                         out[name] = int(s.split()[-1])

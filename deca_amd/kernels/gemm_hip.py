@@ -6,12 +6,14 @@ Counterpart of the reference's src/kernels/gemm_tir.py.  Layout: A[M, K],
 B[K, N], C[M, N], all row-major float16.
 
 What changes on CDNA4 (reference mechanism -> here):
-- mma.sync.m16n8k16 (gemm_tir.py:280-290) -> v_mfma_f32_32x32x16_f16; a wave is
-  64 lanes and owns a `warp_m x warp_n` tile made of 32x32 MFMA tiles;
+- mma.sync.m16n8k16 (gemm_tir.py:280-290) -> v_mfma_f32_32x32x16_f16 or (`mfma=16`)
+  v_mfma_f32_16x16x32_f16; a wave is 64 lanes and owns a `warp_m x warp_n` tile made of
+  32x32 (16x16) MFMA tiles;
 - ldmatrix / ldmatrix.trans (:262-278) -> ds_read_b128 for A and the transposing
   ds_read_b64_tr_b16 for the row-major B tile;
-- cp.async ring (:190-199) -> 16-byte global loads staged through VGPRs one
-  K-tile ahead of the MFMAs, into a 1- or 2-deep LDS ring;
+- cp.async ring (:190-199) -> asynchronous 16-byte global -> LDS loads that bypass the
+  VGPRs (`direct`, ring of 2 to 5 K-tiles, explicit vmcnt waits), or 16-byte global loads
+  staged through VGPRs one K-tile ahead of the MFMAs into a 1- or 2-deep LDS ring;
 - 128-byte-line XOR swizzle (:14-18) -> chunk swizzles sized for the 64-bank LDS;
 - grouped rasterisation (:159-163) -> the same grouping applied after dealing
   contiguous tile ranges to the 8 XCDs (each has a private L2);
@@ -164,6 +166,9 @@ def check_config(cfg: GemmConfig, M: int, N: int, K: int, max_smem: int = MAX_LD
         assert cfg.direct
         assert cfg.BK == 64 or (K // cfg.BK) % 2 == 0
         assert 0 <= cfg.early < cfg.warp_m // 16
+        # 64 accumulator tiles of 16 x 16 per wave: hipcc fills all 256 accumulation and
+        # all 256 vector registers and still spills 30-170 inside the loop (8x slower)
+        assert (cfg.warp_m // 16) * (cfg.warp_n // 16) <= 32
     else:
         assert cfg.early == 0
     assert cfg.warp_m % MFMA_M == 0 and cfg.warp_n % MFMA_M == 0
@@ -234,7 +239,11 @@ def make_gemm_tc(M: int, N: int, K: int, cfg: GemmConfig, dtype: str = "float16"
         workgroups += 3 * r
     return make_spec(
         TEMPLATE, defines, grid=(workgroups, 1, 1), block=(cfg.threads, 1, 1),
-        nargs=3, options=FAST_MATH_OPTIONS, meta={"cfg": str(cfg), "dtype": dtype},
+        nargs=3, options=FAST_MATH_OPTIONS,
+        # the direct-load ring waits with vmcnt(n > 0) once it is deeper than two tiles
+        # (the quarter tiles of `tail` always are): the loader refuses a build that spills
+        meta={"cfg": str(cfg), "dtype": dtype,
+              "no_scratch": bool(cfg.direct and (cfg.stages > 2 or cfg.tail))},
     )
 
 

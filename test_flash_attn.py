@@ -96,6 +96,10 @@ def main(argv=None):
         for (B, H, S_q, _, D), cfg, tflops, sdpa_tflops in summary:
             print(f"{B:>3} {H:>3} {S_q:>6} {D:>4} | {tflops:>7.1f} {sdpa_tflops:>7.1f} "
                   f"{tflops / sdpa_tflops:>6.3f} | {cfg}")
+        from deca_amd.kernels import attn_bench
+
+        print(f"SDPA column: torch.nn.functional.scaled_dot_product_attention, back end: "
+              f"{attn_bench.SDPA_BACKEND}")
     return summary
 
 

@@ -211,5 +211,19 @@ def fa_specs():
             for B, H, Sq, Skv, D, causal, cfg in FA_CASES + FA_FULL]
 
 
+def spilling_specs():
+    """The same code object twice: an attention kernel at D = 320 whose registers do not fit
+    (80 bytes of scratch per lane), plain and marked as one that must not spill.  The kernel
+    only ever waits with vmcnt(0), so it is correct as it is; the mark is what the loader's
+    refusal is tested with."""
+    from deca_amd.kernels.build import make_spec
+
+    plain = make_flash_attn_fwd(1, 2, 256, 256, 320, FAConfig(128, 64, 4, 2), None, False)
+    marked = make_spec(plain.template, dict(plain.defines), plain.grid, plain.block, plain.nargs,
+                       lds_bytes=plain.lds_bytes, options=list(plain.options),
+                       meta=dict(dict(plain.meta), no_scratch=True))
+    return plain, marked
+
+
 def all_specs():
-    return rowwise_specs() + gemm_specs() + fa_specs()
+    return rowwise_specs() + gemm_specs() + fa_specs() + [spilling_specs()[0]]

@@ -112,6 +112,9 @@ def test_fa_score_terms():
     small = FAConfig(128, 64, 4, 2)
     assert (cm.fa_score(small, ARCH, shape, True) / cm.fa_score(small, ARCH, shape)
             < cm.fa_score(b, ARCH, shape, True) / cm.fa_score(b, ARCH, shape))
+    # the 16x16x32 twin of a config ranks just behind it
+    assert cm.fa_score(FAConfig(256, 64, 8, 2, pipe=2, mfma=16), ARCH, shape) == pytest.approx(
+        0.97 * cm.fa_score(FAConfig(256, 64, 8, 2, pipe=2), ARCH, shape))
     wgs, share = cm.fa_occupancy(a, ARCH, 128, 1024)
     assert wgs == 1 and share == pytest.approx(8 / 32)
     assert cm.rank_fa_configs([FAConfig(32, 32, 1, 1), a], ARCH, shape, top_n=1) == [a]

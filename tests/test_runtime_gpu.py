@@ -37,6 +37,30 @@ def test_device_and_function_info(hip):
     kern.close()  # idempotent
 
 
+def test_loader_refuses_a_spilled_kernel_that_was_marked_spill_free():
+    """Kernels that wait for part of their outstanding loads are marked `no_scratch`; a
+    build of such a kernel that spills is refused at load time, not launched."""
+    import kernel_cases
+    from deca_amd.driver.driver import KernelRejected, load_kernel
+    from deca_amd.kernels.attn_bench import make_qkv, math_attention
+    from deca_amd.kernels.build import cached_build
+
+    plain, marked = kernel_cases.spilling_specs()
+    assert plain.key() == marked.key()  # one code object
+    path = cached_build(plain)
+    kern = load_kernel(plain, path)
+    assert kern.info()["scratch_bytes"] > 0
+    # unmarked it loads and is right (it only ever waits for all of its loads)
+    q, k, v = make_qkv(1, 2, 256, 256, 320)
+    o = torch.full_like(q, float("nan"))
+    kern(q, k, v, o)
+    torch.cuda.synchronize()
+    assert (o.float() - math_attention(q, k, v, False)).abs().max().item() <= 2e-3
+    kern.close()
+    with pytest.raises(KernelRejected, match="spills"):
+        load_kernel(marked, path)
+
+
 def test_runtime_mod_rowwise_build_and_time(arch):
     from deca_amd.kernels.rowwise_hip import RowConfig
     from deca_amd.operators import RMSNorm, Softmax
