@@ -225,5 +225,41 @@ def spilling_specs():
     return plain, marked
 
 
+# Shapes whose solver output runs on the GPU config by config (test_all_configs_gpu.py):
+# a sample of SAMPLE evenly spaced configurations each by default.
+SOLVER_FA_SHAPES = [(2, 16, 1024, 64, False), (2, 16, 1024, 64, True), (2, 16, 1024, 128, False),
+                    (2, 16, 1024, 128, True), (1, 16, 2048, 256, True), (2, 16, 1024, 192, False),
+                    (2, 16, 1024, 192, True)]
+SOLVER_GEMM_SHAPES = [(2048, 2048, 2048), (3072, 3072, 512)]  # the second leaves partial waves (tail)
+SOLVER_ROW_SHAPES = [("softmax", 2048, 4096, "float16"), ("rmsnorm", 2048, 8192, "bfloat16"),
+                     ("softmax", 512, 32000, "float16"), ("rmsnorm", 512, 128256, "float16")]
+SAMPLE = 24
+
+
+def solver_sample(configs, n: int = SAMPLE):
+    """`n` evenly spaced entries of a solver's list (all of it when it is shorter)."""
+    if len(configs) <= n:
+        return list(configs)
+    return [configs[(i * len(configs)) // n] for i in range(n)]
+
+
+def solver_sample_specs():
+    from deca_amd import Solver
+    from deca_amd.arch.MI355X import MI355X
+
+    arch = MI355X()
+    specs = []
+    for B, H, S, D, causal in SOLVER_FA_SHAPES:
+        specs += [make_flash_attn_fwd(B, H, S, S, D, cfg, None, causal)
+                  for cfg in solver_sample(Solver.solve_flash_attn(arch, B, H, S, S, D))]
+    for M, N, K in SOLVER_GEMM_SHAPES:
+        specs += [make_gemm_tc(M, N, K, cfg) for cfg in solver_sample(Solver.solve_gemm_tc(arch, M, N, K))]
+    for op, M, N, dtype in SOLVER_ROW_SHAPES:
+        specs += [make_rowwise(op, M, N, dtype, cfg, 1e-6)
+                  for cfg in solver_sample(Solver.solve_rowwise(arch, op, M, N))]
+    return specs
+
+
 def all_specs():
-    return rowwise_specs() + gemm_specs() + fa_specs() + [spilling_specs()[0]]
+    return (rowwise_specs() + gemm_specs() + fa_specs() + [spilling_specs()[0]]
+            + solver_sample_specs())

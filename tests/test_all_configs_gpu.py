@@ -1,9 +1,11 @@
-"""Every configuration the solvers emit for a few small shapes, run once on the
-GPU against torch's fp32 result of the same operator.
+"""Configurations the solvers emit for a few small shapes, run once on the GPU against
+torch's fp32 result of the same operator.
 
-This compiles several hundred code objects (minutes of host time), so it only
-runs when DECA_ALL_CONFIGS=1 is set; the regular GPU suite covers a hand-picked
-subset (kernel_cases.py).  Gates are the ones of the other GPU tests.
+By default an evenly spaced sample of each solver's list runs (SAMPLE configurations per
+shape; `kernel_cases.all_specs()` names the same kernels, so the build step compiles them
+beforehand).  With DECA_ALL_CONFIGS=1 every configuration runs (every GEMM_STRIDE-th for the
+GEMM): several thousand code objects, minutes of host time to compile.  Gates are the ones of
+the other GPU tests.
 """
 
 import os
@@ -12,18 +14,12 @@ from concurrent.futures import ThreadPoolExecutor
 import pytest
 import torch
 
-pytestmark = [
-    pytest.mark.gpu,
-    pytest.mark.skipif(os.environ.get("DECA_ALL_CONFIGS") != "1",
-                       reason="opt-in: compiles every solver configuration (set DECA_ALL_CONFIGS=1)"),
-]
+from kernel_cases import (SOLVER_FA_SHAPES as FA_SHAPES, SOLVER_GEMM_SHAPES as GEMM_SHAPES,
+                          SOLVER_ROW_SHAPES as ROW_SHAPES, solver_sample)
 
-FA_SHAPES = [(2, 16, 1024, 64, False), (2, 16, 1024, 64, True), (2, 16, 1024, 128, False),
-             (2, 16, 1024, 128, True), (1, 16, 2048, 256, True), (2, 16, 1024, 192, False),
-             (2, 16, 1024, 192, True)]
-GEMM_SHAPES = [(2048, 2048, 2048), (3072, 3072, 512)]  # the second leaves partial waves (tail)
-ROW_SHAPES = [("softmax", 2048, 4096, "float16"), ("rmsnorm", 2048, 8192, "bfloat16"),
-              ("softmax", 512, 32000, "float16"), ("rmsnorm", 512, 128256, "float16")]
+pytestmark = [pytest.mark.gpu]
+
+EVERY = os.environ.get("DECA_ALL_CONFIGS") == "1"
 GEMM_STRIDE = int(os.environ.get("DECA_ALL_CONFIGS_GEMM_STRIDE", "7"))  # 1: every GEMM config
 GEMM_MFMA = os.environ.get("DECA_ALL_CONFIGS_GEMM_MFMA")  # "16" / "32": only that MFMA tile form
 
@@ -32,6 +28,8 @@ def gemm_configs(M, N, K):
     from deca_amd import Solver
 
     configs = Solver.solve_gemm_tc(_arch(), M, N, K)
+    if not EVERY:
+        return solver_sample(configs)
     if GEMM_MFMA:
         configs = [c for c in configs if c.mfma == int(GEMM_MFMA)]
     return configs[::GEMM_STRIDE]
@@ -75,6 +73,8 @@ def test_every_flash_attn_config(B, H, S, D, causal):
     from deca_amd.kernels.flash_attn_hip import make_flash_attn_fwd
 
     configs = Solver.solve_flash_attn(_arch(), B, H, S, S, D)
+    if not EVERY:
+        configs = solver_sample(configs)
     specs = [make_flash_attn_fwd(B, H, S, S, D, cfg, None, causal) for cfg in configs]
     paths = _build_all(specs)
     q, k, v = make_qkv(B, H, S, S, D)
@@ -126,6 +126,8 @@ def test_every_rowwise_config(op, M, N, dtype):
     from deca_amd.kernels.rowwise_hip import make_rowwise
 
     configs = Solver.solve_rowwise(_arch(), op, M, N)
+    if not EVERY:
+        configs = solver_sample(configs)
     specs = [make_rowwise(op, M, N, dtype, cfg, 1e-6) for cfg in configs]
     paths = _build_all(specs)
     inputs = make_inputs(op, M, N, dtype, std=2.0 if op == "softmax" else 1.0)
