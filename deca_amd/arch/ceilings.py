@@ -130,6 +130,25 @@ def measure_streams(out=sys.stdout):
               file=out, flush=True)
 
 
+def run_copy(launches: int = 16, out=sys.stdout):
+    """Only the plain copy (512 lanes, non-temporal, one 16-byte access per lane), `launches`
+    times over rotating 128 MiB buffers: the kernel of known traffic that the L2 <-> fabric
+    counters of rocprofv3 (FETCH_SIZE, WRITE_SIZE) are scaled against."""
+    import torch
+
+    from deca_amd.driver.driver import load_kernel
+
+    n = STREAM_BYTES // 4
+    bufs = [(torch.randn(n, device="cuda"), torch.empty(n, device="cuda")) for _ in range(ROTATE)]
+    spec = stream_spec(0, 512, 1, 1, 0)
+    kern = load_kernel(spec, cached_build(spec))
+    for i in range(launches):
+        kern(*bufs[i % ROTATE])
+    torch.cuda.synchronize()
+    assert torch.equal(bufs[0][0], bufs[0][1])
+    print(f"copy: {launches} launches of {STREAM_BYTES} bytes in, {STREAM_BYTES} bytes out", file=out, flush=True)
+
+
 def measure_lds(out=sys.stdout):
     """Bytes per nominal 2.4 GHz clock and CU (these loops draw little power: the shader
     clock stays at its maximum)."""
@@ -274,9 +293,14 @@ def main(argv=None):
     ap = argparse.ArgumentParser()
     ap.add_argument("--build", action="store_true", help="compile the probe kernels and exit")
     ap.add_argument("--sclk", action="store_true", help="also sample the shader clock under the GEMM")
+    ap.add_argument("--copy-only", action="store_true",
+                    help="run only the plain copy kernel (the calibration target of the traffic counters)")
     args = ap.parse_args(argv)
     build()
     if args.build:
+        return
+    if args.copy_only:
+        run_copy()
         return
     measure_streams()
     measure_lds()
