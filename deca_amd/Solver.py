@@ -470,6 +470,17 @@ def solve_flash_attn(arch, B: int, H: int, S_q: int, S_kv: int, D: int, type_siz
 
     if D % 64 != 0 or D < 64:  # flash_attn_tir.py:70-72
         return []
+    from dataclasses import replace
+
+    from deca_amd.kernels.flash_attn_hip import register_fill
+
     cons = _fa_constraints(arch, B, H, S_q, S_kv, D, type_size, max_est_regs)
-    return [FAConfig(Br=br, Bc=bc, num_warps=nw, stages=st, pipe=int(pipe), mfma=mfma)
-            for br, bc, nw, st, pipe, mfma in _enumerate(FA_DOMAINS, cons, count, backend)]
+    results = []
+    for br, bc, nw, st, pipe, mfma in _enumerate(FA_DOMAINS, cons, count, backend):
+        cfg = FAConfig(Br=br, Bc=bc, num_warps=nw, stages=st, pipe=int(pipe), mfma=mfma)
+        results.append(cfg)
+        # the plain two-stage loop in its one-copy form, where the unrolled one is expected to
+        # run out of registers (it interacts with no other constraint: expanded here)
+        if int(pipe) == 0 and st == 2 and register_fill(cfg, D) >= 0.95:
+            results.append(replace(cfg, roll=True))
+    return results

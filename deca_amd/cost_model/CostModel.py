@@ -326,6 +326,11 @@ def fa_score(cfg, arch, shape, causal: bool = False) -> float:
     # ahead of it under the causal mask at D = 128 (the twins stay tied there).
     if getattr(cfg, "mfma", 32) == 16 and not causal:
         pipe *= 0.97
+    # one copy of the two-stage plain loop: no overlap between the end of a step and the start
+    # of the next (measured 1-10 % behind the unrolled form where that fits its registers; the
+    # solver only emits it where the unrolled form is expected to spill)
+    if getattr(cfg, "roll", False):
+        pipe *= 0.99
     sync = 1.0 / (1.0 + getattr(arch, "fa_cta_sync_penalty", 0.0) * cfg.num_warps / 4 / wgs)
     # longer KV steps amortise the per-step max / barrier; the slot loop has the row
     # statistics inside the matrix work and pays a little less of it

@@ -66,6 +66,9 @@
 #ifndef DECA_EPI_LDS
 #define DECA_EPI_LDS 1
 #endif
+#ifndef DECA_ROLL
+#define DECA_ROLL 0  // plain loop with two LDS stages: 1 keeps a single copy of the step
+#endif
 #ifndef DECA_MIN_WAVES
 #define DECA_MIN_WAVES 1  // waves per SIMD the register allocation must leave room for
 #endif
@@ -969,7 +972,11 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
 #else
   issue_k(0, 0);
   issue_v(0, 0);
-#if STAGES == 2
+#if STAGES == 2 && DECA_ROLL
+  // one copy of the step, the ring slot a run-time value
+#pragma unroll 1
+  for (int j = 0; j < nkv; ++j) kv_step(j, j & 1);
+#elif STAGES == 2
   for (int j = 0; j < nkv; j += 2) {
     kv_step(j, 0);
     if (j + 1 < nkv) kv_step(j + 1, 1);

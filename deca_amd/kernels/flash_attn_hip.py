@@ -46,6 +46,11 @@ class FAConfig:
     pipe: int = 0
     # MFMA tile: 32 -> v_mfma_f32_32x32x16, 16 -> v_mfma_f32_16x16x32 (plain and slot loop)
     mfma: int = 32
+    # Plain loop over two LDS stages: False unrolls it by two (each copy of the step knows its
+    # ring slot and the scheduler overlaps the end of one step with the start of the next),
+    # True keeps one copy with the slot as a run-time value (about 50 registers fewer: for
+    # the tiles whose unrolled loop does not fit the register file of two waves per SIMD).
+    roll: bool = False
 
     @property
     def threads(self) -> int:
@@ -60,6 +65,7 @@ class FAConfig:
             f"q_smem={int(self.q_in_smem)},swz={int(self.swizzle)}"
             + (f",pipe={int(self.pipe)}" if self.pipe else "")
             + (f",mfma={self.mfma}" if self.mfma != 32 else "")
+            + (",roll=1" if self.roll else "")
         )
 
 
@@ -97,6 +103,13 @@ def expect_spill_free(cfg: FAConfig, D: int) -> bool:
     """Whether the compiler is expected to fit the kernel's registers (see above)."""
     limit = SPILL_FREE_EST_REGS.get((int(cfg.pipe), cfg.stages))
     return limit is not None and est_regs_per_thread(cfg, D) <= limit
+
+
+def register_fill(cfg: FAConfig, D: int) -> float:
+    """Estimated registers as a share of what a wave gets at the occupancy the kernel is
+    compiled for.  From about 0.95 the unrolled two-stage plain loop spills (measured:
+    D = 128, Br=256, Bc=128, 8 waves: 0.98, 3 to 67 spilled registers; rolled: none)."""
+    return est_regs_per_thread(cfg, D) / (512 / target_waves_per_simd(cfg, D))
 
 
 def target_waves_per_simd(cfg: FAConfig, D: int) -> int:
@@ -153,6 +166,7 @@ def check_config(cfg: FAConfig, S_q: int, S_kv: int, D: int) -> None:
     assert cfg.mfma in (32, 16)
     assert cfg.mfma == 32 or int(cfg.pipe) != 1, "the 16x16x32 form exists for the plain and the slot loop"
     assert not cfg.pipe or cfg.stages == 2
+    assert not cfg.roll or (int(cfg.pipe) == 0 and cfg.stages == 2), "roll is a form of the plain two-stage loop"
     assert int(cfg.pipe) != 2 or slot_schedule_ok(cfg.Bc, D, cfg.mfma)
     assert not cfg.q_in_smem and cfg.swizzle
     assert smem_bytes(cfg, D) <= MAX_LDS
@@ -186,6 +200,8 @@ def make_flash_attn_fwd(
     }
     if cfg.mfma == 16:
         defines["DECA_MFMA16"] = 1
+    if cfg.roll:
+        defines["DECA_ROLL"] = 1
     return make_spec(
         TEMPLATE, defines, grid=((S_q // cfg.Br) * B * H, 1, 1), block=(cfg.threads, 1, 1), nargs=4,
         options=FAST_MATH_OPTIONS, meta={"cfg": str(cfg), "causal": causal},

@@ -192,6 +192,12 @@ FA_CASES = [
     (1, 2, 512, 512, 192, False, FAConfig(128, 64, 4, 2, pipe=2)),
     (1, 2, 512, 512, 192, True, FAConfig(128, 64, 4, 2, pipe=2)),
     (1, 1, 256, 256, 320, True, FAConfig(32, 32, 1, 2)),
+    # the plain two-stage loop as one copy of the step (run-time ring slot): both tile
+    # forms, full and causal, an odd number of KV tiles
+    (1, 2, 512, 512, 128, False, FAConfig(256, 128, 8, 2, mfma=16, roll=True)),
+    (1, 2, 512, 512, 128, True, FAConfig(256, 128, 8, 2, roll=True)),
+    (2, 2, 256, 320, 64, False, FAConfig(128, 64, 4, 2, roll=True)),
+    (1, 2, 512, 512, 64, True, FAConfig(128, 64, 4, 2, mfma=16, roll=True)),
 ]
 
 FA_FULL = [

@@ -4,6 +4,7 @@ independent filter over the raw domain product), and the documented rules
 (reg vs twopass, raster / XCD expansion) hold."""
 
 import itertools
+from dataclasses import replace
 
 import pytest
 
@@ -153,6 +154,9 @@ def test_flash_attn_configs_are_valid(D, S):
         if regs * -(-nw // 4) > 512 or not fa.expect_spill_free(cfg, D):
             continue
         want.add(cfg)
+        # the one-copy form of the plain two-stage loop, where the unrolled one is tight
+        if pipe == 0 and st == 2 and fa.register_fill(cfg, D) >= 0.95:
+            want.add(replace(cfg, roll=True))
     assert set(configs) == want
     # a tighter register budget removes the widest per-wave tiles
     tight = Solver.solve_flash_attn(ARCH, B, H, S, S, D, max_est_regs=256)
@@ -232,6 +236,17 @@ def test_kernels_are_compiled_for_the_occupancy_the_estimates_allow():
     assert gm.target_waves_per_simd(big) == 2
     assert gm.target_waves_per_simd(gm.GemmConfig(128, 256, 64, 64, 128, 2, 8, True, True, True)) == 1
     assert dict(gm.make_gemm_tc(4096, 4096, 4096, big).defines)["DECA_MIN_WAVES"] == 2
+
+
+def test_flash_attn_rolled_loop_is_offered_where_registers_are_tight():
+    cfgs = Solver.solve_flash_attn(ARCH, 4, 16, 4096, 4096, 128)
+    rolled = {c for c in cfgs if c.roll}
+    assert fa.FAConfig(256, 128, 8, 2, mfma=16, roll=True) in rolled
+    assert all(",roll=1" in str(c) and replace(c, roll=False) in cfgs for c in rolled)
+    assert fa.FAConfig(256, 64, 8, 2, roll=True) not in rolled  # 204 of 256 registers: room enough
+    assert dict(fa.make_flash_attn_fwd(4, 16, 4096, 4096, 128, next(iter(rolled))).defines)["DECA_ROLL"] == 1
+    with pytest.raises(AssertionError):
+        fa.check_config(fa.FAConfig(256, 64, 8, 2, pipe=2, roll=True), 4096, 4096, 128)
 
 
 def test_flash_attn_head_dims():

@@ -263,6 +263,7 @@ def test_config_strings_parse_back():
         ("rmsnorm", RowConfig(1024, 1, 4, "twopass", 4)),
         ("flash_attn", FAConfig(256, 64, 8, 2, pipe=2)),
         ("flash_attn", FAConfig(128, 128, 4, 1)),
+        ("flash_attn", FAConfig(256, 128, 8, 2, mfma=16, roll=True)),
     ]
     for op, cfg in cases:
         assert tuned.parse_config(op, str(cfg)) == cfg
