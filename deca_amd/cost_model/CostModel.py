@@ -234,7 +234,14 @@ def gemm_tc_score(cfg, arch, M: int, N: int, K: int) -> float:
     # MFMA issue stream (measured ~15% on MI355X)
     staged = 1.0 if cfg.direct else getattr(arch, "gemm_staged_fill_factor", 0.85)
 
-    return wave_eff * hiding * pipe * sync_eff * staged / ((t_flop + t_epi) / t_mma)
+    # 16x16x32 tiles: measured ahead of the 32x32x16 twin where the grid is a single wave of
+    # workgroups or leaves a partial one (2048^3 +7 %, 4096^3 +4.5 %, 6144^3 / 10240^3 +2 %),
+    # level with it on the large grids; the barrier inside the last k-step adds a little
+    form = 1.0
+    if getattr(cfg, "mfma", 32) == 16:
+        form = 1.02 + (0.004 if getattr(cfg, "early", 0) else 0.0)
+
+    return form * wave_eff * hiding * pipe * sync_eff * staged / ((t_flop + t_epi) / t_mma)
 
 
 def rank_gemm_configs(configs, arch, M: int, N: int, K: int, top_n: int | None = None,
@@ -320,17 +327,25 @@ def fa_score(cfg, arch, shape, causal: bool = False) -> float:
     # chain for nothing in return (measured 2-8 % behind the plain loop of the same tile)
     if int(cfg.pipe) == 1:
         pipe *= 0.90
-    # 16x16x32 tiles: twice the matrix instructions and LDS fragment reads per FLOP for
-    # the same vector work.  Measured 0-3 % behind the 32x32x16 twin on full shapes (ranked
-    # just behind it there, so that the twins do not fill the measured top-N) and 2-8 %
-    # ahead of it under the causal mask at D = 128 (the twins stay tied there).
-    if getattr(cfg, "mfma", 32) == 16 and not causal:
-        pipe *= 0.97
+    # 16x16x32 tiles, measured against the 32x32x16 twin (S = 4096): slot loop 1-2 % behind
+    # on full shapes and level under the causal mask; plain loop 5-8 % ahead at D = 128 and
+    # 1-2 % behind at D = 64.
+    if getattr(cfg, "mfma", 32) == 16:
+        if int(cfg.pipe) == 2:
+            pipe *= 0.98 if not causal else 1.0
+        else:
+            pipe *= 1.04 if D >= 128 else 0.985
     # one copy of the two-stage plain loop: no overlap between the end of a step and the start
     # of the next (measured 1-10 % behind the unrolled form where that fits its registers; the
     # solver only emits it where the unrolled form is expected to spill)
     if getattr(cfg, "roll", False):
         pipe *= 0.99
+    elif int(cfg.pipe) == 0 and cfg.stages == 2:
+        from deca_amd.kernels.flash_attn_hip import register_fill
+
+        # the unrolled form of a tile this tight is expected to spill (3-67 registers measured)
+        if register_fill(cfg, D) >= 0.95:
+            pipe *= 0.9
     sync = 1.0 / (1.0 + getattr(arch, "fa_cta_sync_penalty", 0.0) * cfg.num_warps / 4 / wgs)
     # longer KV steps amortise the per-step max / barrier; the slot loop has the row
     # statistics inside the matrix work and pays a little less of it

@@ -112,9 +112,13 @@ def test_fa_score_terms():
     small = FAConfig(128, 64, 4, 2)
     assert (cm.fa_score(small, ARCH, shape, True) / cm.fa_score(small, ARCH, shape)
             < cm.fa_score(b, ARCH, shape, True) / cm.fa_score(b, ARCH, shape))
-    # the 16x16x32 twin of a config ranks just behind it
+    # 16x16x32 tiles: just behind the 32x32x16 twin in the slot loop, ahead of it in the plain
+    # loop at D = 128, behind it at D = 64 (as measured)
     assert cm.fa_score(FAConfig(256, 64, 8, 2, pipe=2, mfma=16), ARCH, shape) == pytest.approx(
-        0.97 * cm.fa_score(FAConfig(256, 64, 8, 2, pipe=2), ARCH, shape))
+        0.98 * cm.fa_score(FAConfig(256, 64, 8, 2, pipe=2), ARCH, shape))
+    assert cm.fa_score(FAConfig(256, 64, 8, 2, mfma=16), ARCH, shape) > cm.fa_score(FAConfig(256, 64, 8, 2), ARCH, shape)
+    d64 = (4, 16, 4096, 4096, 64)
+    assert cm.fa_score(FAConfig(256, 64, 4, 2, mfma=16), ARCH, d64) < cm.fa_score(FAConfig(256, 64, 4, 2), ARCH, d64)
     wgs, share = cm.fa_occupancy(a, ARCH, 128, 1024)
     assert wgs == 1 and share == pytest.approx(8 / 32)
     assert cm.rank_fa_configs([FAConfig(32, 32, 1, 1), a], ARCH, shape, top_n=1) == [a]
