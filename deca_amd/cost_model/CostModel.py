@@ -345,7 +345,7 @@ def fa_score(cfg, arch, shape, causal: bool = False) -> float:
 
         # the unrolled form of a tile this tight is expected to spill (3-67 registers measured)
         if register_fill(cfg, D) >= 0.95:
-            pipe *= 0.9
+            pipe *= 0.965
     sync = 1.0 / (1.0 + getattr(arch, "fa_cta_sync_penalty", 0.0) * cfg.num_warps / 4 / wgs)
     # longer KV steps amortise the per-step max / barrier; the slot loop has the row
     # statistics inside the matrix work and pays a little less of it
