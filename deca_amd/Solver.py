@@ -351,7 +351,7 @@ def solve_gemm_tc(arch, M: int, N: int, K: int, type_size: int = 2, count: int =
     """
     from dataclasses import replace
 
-    from deca_amd.kernels.gemm_hip import GemmConfig, check_config
+    from deca_amd.kernels.gemm_hip import GemmConfig, agpr_split_fits, check_config
 
     tiles = _enumerate(GEMM_DOMAINS, _gemm_constraints(arch, M, N, K, type_size), count, backend)
     results = []
@@ -372,6 +372,10 @@ def solve_gemm_tc(arch, M: int, N: int, K: int, type_size: int = 2, count: int =
             if mfma == 16 and wm >= 64:
                 # the barrier of a K-tile after half of the row blocks of its last k-step
                 cands += [replace(c, early=wm // 32) for c in cands]
+            if mfma == 16:
+                # the accumulators in accumulation registers, where both halves of the
+                # register file have room for their share
+                cands += [replace(c, agpr=True) for c in cands if agpr_split_fits(c)]
             for cand in cands:
                 if ras == 0 or cand.tail:
                     try:

@@ -62,6 +62,9 @@
 #ifndef DECA_MFMA16
 #define DECA_MFMA16 0  // 1: v_mfma_f32_16x16x32 tiles instead of 32x32x16
 #endif
+#ifndef DECA_ACC_AGPR
+#define DECA_ACC_AGPR 0  // 16x16x32 body: 1 keeps the accumulators in accumulation registers (MFMAs as inline asm)
+#endif
 #ifndef DECA_EARLY_GROUPS
 #define DECA_EARLY_GROUPS 0  // 16x16x32 body: MFMA groups of a K-tile's last k-step issued before its barrier
 #endif
@@ -69,6 +72,7 @@
 typedef __bf16 elem_t;
 #if DECA_MFMA16
 #define DECA_MFMA __builtin_amdgcn_mfma_f32_16x16x32_bf16
+#define DECA_MFMA_ASM "v_mfma_f32_16x16x32_bf16"
 #else
 #define DECA_MFMA __builtin_amdgcn_mfma_f32_32x32x16_bf16
 #endif
@@ -76,6 +80,7 @@ typedef __bf16 elem_t;
 typedef _Float16 elem_t;
 #if DECA_MFMA16
 #define DECA_MFMA __builtin_amdgcn_mfma_f32_16x16x32_f16
+#define DECA_MFMA_ASM "v_mfma_f32_16x16x32_f16"
 #else
 #define DECA_MFMA __builtin_amdgcn_mfma_f32_32x32x16_f16
 #endif

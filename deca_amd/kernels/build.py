@@ -118,23 +118,64 @@ def compile_command(spec: KernelSpec, arch: str, out_path: str) -> list[str]:
     ]
 
 
+def check_generated_code(spec: KernelSpec, asm_text: str) -> None:
+    """What a spec promises about its generated ISA (`meta`), checked on the assembly text.
+
+    `accumulator_moves`: the kernel keeps MFMA accumulators in accumulation registers through
+    inline assembly, with the wait states around them placed by hand.  That is only valid
+    while the compiler never touches an accumulator between its initialisation and the
+    epilogue, so the number of `v_accvgpr_*` instructions must be exactly the promised one
+    and nothing may spill."""
+    meta = dict(spec.meta)
+    want = meta.get("accumulator_moves")
+    if want is None:
+        return
+    got = len(re.findall(r"^\s*v_accvgpr_(?:read|write|mov)_b32", asm_text, re.M))
+    spills = [int(v) for v in re.findall(r"\.vgpr_spill_count:\s*(\d+)", asm_text)]
+    scratch = [int(v) for v in re.findall(r"\.private_segment_fixed_size:\s*(\d+)", asm_text)]
+    if got != want or any(spills) or any(scratch):
+        raise RuntimeError(
+            f"{spec.template} [{meta.get('cfg', '')}]: {got} accumulation-register moves where "
+            f"{want} are accounted for, {sum(spills)} spilled registers: the compiler moves "
+            "accumulators it cannot know to be in flight")
+
+
 def build_kernel(spec: KernelSpec, arch: str | None, path: str, dump_dir: str | None = None) -> str:
     """Compiles `spec` into the code object `path`; `dump_dir` keeps the
-    generated ISA (`*.s`) for inspection (reference: build.py:73-87)."""
+    generated ISA (`*.s`) for inspection (reference: build.py:73-87).  A spec that makes
+    promises about its generated code (`check_generated_code`) is compiled with the ISA
+    kept and refused when they do not hold."""
     arch = arch or DEFAULT_ARCH
     os.makedirs(os.path.dirname(os.path.abspath(path)) or ".", exist_ok=True)
     tmp = f"{path}.tmp{os.getpid()}_{threading.get_ident()}"
     cmd = compile_command(spec, arch, tmp)
-    cwd = None
+    cwd, scratch_dir = None, None
+    checked = "accumulator_moves" in dict(spec.meta)
     if dump_dir:
         os.makedirs(dump_dir, exist_ok=True)
-        cmd.append("--save-temps")
         cwd = dump_dir
-    proc = subprocess.run(cmd, capture_output=True, text=True, cwd=cwd)
-    if proc.returncode != 0:
+    elif checked:
+        scratch_dir = tempfile.mkdtemp(prefix="deca_isa_")
+        cwd = scratch_dir
+    if cwd:
+        cmd.append("--save-temps")
+    try:
+        proc = subprocess.run(cmd, capture_output=True, text=True, cwd=cwd)
+        if proc.returncode != 0:
+            raise RuntimeError(f"hipcc failed for {spec.show()}:\n{proc.stderr[-4000:]}")
+        if checked:
+            texts = [open(os.path.join(cwd, f)).read() for f in sorted(os.listdir(cwd))
+                     if f.endswith(".s") and "amdgcn" in f]
+            if not texts:
+                raise RuntimeError(f"no device assembly was kept for {spec.show()}")
+            check_generated_code(spec, texts[-1])
+    except Exception:
         if os.path.exists(tmp):
             os.remove(tmp)
-        raise RuntimeError(f"hipcc failed for {spec.show()}:\n{proc.stderr[-4000:]}")
+        raise
+    finally:
+        if scratch_dir:
+            shutil.rmtree(scratch_dir, ignore_errors=True)
     os.replace(tmp, path)
     return path
 

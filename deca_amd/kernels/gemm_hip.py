@@ -64,6 +64,10 @@ class GemmConfig:
     # barrier which publishes the next tile (a later barrier gives the loads more time,
     # and leaves fewer MFMAs to cover the first fragment reads of the next tile)
     early: int = 0
+    # 16x16x32 body: accumulators tied to accumulation registers (AGPRs), the MFMAs written
+    # as inline assembly (about 3 % faster than the builtin form; the build step checks the
+    # generated code, see `accumulator_moves`)
+    agpr: bool = False
 
     @property
     def num_warps(self) -> int:
@@ -85,6 +89,7 @@ class GemmConfig:
             + (",tail=1" if self.tail else "")
             + (f",mfma={self.mfma}" if self.mfma != 32 else "")
             + (f",early={self.early}" if self.early else "")
+            + (",agpr=1" if self.agpr else "")
         )
 
 
@@ -144,6 +149,27 @@ def tail_stages(cfg: GemmConfig) -> int:
     return min(4 if cfg.direct else 2, 2 * cfg.stages)
 
 
+def agpr_split_fits(cfg: GemmConfig) -> bool:
+    """Whether the 16x16x32 body is expected to build with its accumulators in accumulation
+    registers: the compiler then gives each half of the register file half of a wave's
+    budget, so the accumulators and everything else must each fit their half."""
+    acc = (cfg.warp_m // 16) * (cfg.warp_n // 16) * 4
+    half = (512 // target_waves_per_simd(cfg)) // 2
+    return cfg.mfma == 16 and acc <= half and est_regs_per_thread(cfg) - acc <= half - 8
+
+
+def accumulator_moves(cfg: GemmConfig) -> int:
+    """`v_accvgpr_*` instructions a kernel with `agpr` accumulators may contain: one write per
+    accumulator register to clear it and one read in the epilogue, for the full tile and,
+    with `tail`, for the quarter tile.  The compiler does not know that the asm statements
+    are matrix instructions and would not wait for one before it moves an accumulator; a
+    build with any further move is refused (`build.check_generated_code`)."""
+    regs = (cfg.warp_m // 16) * (cfg.warp_n // 16) * 4
+    if cfg.tail:
+        regs += (cfg.warp_m // 32) * (cfg.warp_n // 32) * 4
+    return 2 * regs
+
+
 def target_waves_per_simd(cfg: GemmConfig) -> int:
     """Waves per SIMD the kernel is compiled for: what the estimated registers and the LDS
     footprint let co-reside.  The compiler only knows the block size, and gives a workgroup
@@ -170,7 +196,7 @@ def check_config(cfg: GemmConfig, M: int, N: int, K: int, max_smem: int = MAX_LD
         # all 256 vector registers and still spills 30-170 inside the loop (8x slower)
         assert (cfg.warp_m // 16) * (cfg.warp_n // 16) <= 32
     else:
-        assert cfg.early == 0
+        assert cfg.early == 0 and not cfg.agpr
     assert cfg.warp_m % MFMA_M == 0 and cfg.warp_n % MFMA_M == 0
     assert cfg.BM % cfg.warp_m == 0 and cfg.BN % cfg.warp_n == 0
     assert cfg.BN >= 64
@@ -231,6 +257,8 @@ def make_gemm_tc(M: int, N: int, K: int, cfg: GemmConfig, dtype: str = "float16"
     if cfg.mfma == 16:
         defines["DECA_MFMA16"] = 1
         defines["DECA_EARLY_GROUPS"] = cfg.early
+    if cfg.agpr:
+        defines["DECA_ACC_AGPR"] = 1
     workgroups = (M // cfg.BM) * (N // cfg.BN)
     if cfg.tail:
         r = tail_tiles(cfg, M, N)
@@ -243,7 +271,8 @@ def make_gemm_tc(M: int, N: int, K: int, cfg: GemmConfig, dtype: str = "float16"
         # the direct-load ring waits with vmcnt(n > 0) once it is deeper than two tiles
         # (the quarter tiles of `tail` always are): the loader refuses a build that spills
         meta={"cfg": str(cfg), "dtype": dtype,
-              "no_scratch": bool(cfg.direct and (cfg.stages > 2 or cfg.tail))},
+              "no_scratch": bool(cfg.direct and (cfg.stages > 2 or cfg.tail)),
+              **({"accumulator_moves": accumulator_moves(cfg)} if cfg.agpr else {})},
     )
 
 

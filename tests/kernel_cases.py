@@ -99,6 +99,14 @@ GEMM_CASES = [
     (3072, 4096, 128, GemmConfig(128, 128, 64, 64, 64, 2, 0, False, True, True, mfma=16, early=2)),
     (3072, 3072, 256, GemmConfig(128, 128, 64, 64, 64, 2, 0, True, True, True, True, mfma=16)),
     (3072, 3072, 256, GemmConfig(128, 128, 64, 64, 64, 2, 4, True, True, True, True, mfma=16, early=2)),
+    # ... with the accumulators tied to accumulation registers: the large and the small wave
+    # tiles, one k-step per K-tile, deep rings, the barrier inside the last k-step, the tail
+    (512, 512, 512, GemmConfig(256, 256, 64, 128, 64, 2, 1, True, False, True, mfma=16, agpr=True)),
+    (512, 512, 512, GemmConfig(256, 256, 64, 128, 64, 2, 2, False, False, True, mfma=16, early=4, agpr=True)),
+    (512, 1024, 256, GemmConfig(128, 128, 32, 64, 32, 4, 2, True, True, True, mfma=16, agpr=True)),
+    (384, 640, 1088, GemmConfig(128, 128, 64, 64, 32, 5, 1, True, False, True, mfma=16, early=2, agpr=True)),
+    (256, 256, 128, GemmConfig(64, 64, 64, 32, 32, 2, 1, False, False, True, mfma=16, agpr=True)),
+    (3072, 3072, 256, GemmConfig(128, 128, 64, 64, 64, 2, 0, True, True, True, True, mfma=16, agpr=True)),
     # VGPR-staged ring
     (3840, 3840, 128, GemmConfig(128, 128, 64, 64, 64, 1, 2, True, True, False, True)),  # tail
     (512, 512, 512, GemmConfig(256, 256, 64, 128, 128, 2, 1, False, False, False)),
@@ -115,6 +123,7 @@ GEMM_FULL = [
     (8192, 8192, 8192, GemmConfig(256, 256, 64, 128, 64, 2, 0, True, True, True)),
     (6144, 6144, 6144, GemmConfig(256, 256, 64, 128, 64, 2, 8, True, True, True, True)),
     (8192, 8192, 8192, GemmConfig(256, 256, 64, 128, 64, 2, 0, True, True, True, mfma=16, early=4)),
+    (8192, 8192, 8192, GemmConfig(256, 256, 64, 128, 64, 2, 0, True, True, True, mfma=16, early=4, agpr=True)),
 ]
 
 
@@ -126,6 +135,7 @@ GEMM_BF16_CASES = [
     (3072, 3072, 256, GemmConfig(128, 128, 64, 64, 64, 2, 0, True, True, True, True)),  # block order + tail
     (512, 512, 512, GemmConfig(256, 256, 64, 128, 64, 2, 1, True, False, True, mfma=16, early=4)),
     (512, 1024, 256, GemmConfig(128, 128, 32, 64, 64, 3, 2, False, True, True, mfma=16)),
+    (512, 512, 512, GemmConfig(256, 256, 64, 128, 64, 2, 1, True, False, True, mfma=16, agpr=True)),
 ]
 
 

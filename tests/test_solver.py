@@ -262,6 +262,24 @@ def test_flash_attn_head_dims():
         fa.check_config(fa.FAConfig(128, 64, 4, 2), 2048, 2048, 96)
 
 
+def test_gemm_accumulation_register_twins():
+    """16x16x32 configs whose registers split evenly between the two halves of the file come
+    with an `agpr=1` twin; nothing else does."""
+    cfgs = Solver.solve_gemm_tc(ARCH, 4096, 4096, 4096)
+    twins = [c for c in cfgs if c.agpr]
+    assert twins and all(c.mfma == 16 and ",agpr=1" in str(c) and replace(c, agpr=False) in cfgs
+                         and gm.agpr_split_fits(c) for c in twins)
+    big = gm.GemmConfig(256, 256, 64, 128, 64, 2, 0, True, True, True, mfma=16, early=4, agpr=True)
+    assert big in twins
+    spec = gm.make_gemm_tc(4096, 4096, 4096, big)
+    assert dict(spec.defines)["DECA_ACC_AGPR"] == 1
+    # 128 accumulators cleared once and read once
+    assert dict(spec.meta)["accumulator_moves"] == 2 * 128 == gm.accumulator_moves(big)
+    assert gm.accumulator_moves(replace(big, tail=True)) == 2 * (128 + 32)
+    with pytest.raises(AssertionError):
+        gm.check_config(replace(big, mfma=32, early=0), 4096, 4096, 4096)
+
+
 def test_gemm_tail_split_is_offered_where_a_partial_wave_remains():
     """6144^3 with 256 x 256 tiles: 576 tiles = 2 waves of 256 + 64; the 64 may run as 256
     quarter tiles.  A grid that fills its waves exactly gets no such variant."""

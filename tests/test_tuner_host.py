@@ -258,6 +258,7 @@ def test_config_strings_parse_back():
     cases = [
         ("GEMM", GemmConfig(256, 256, 64, 128, 64, 2, 0, True, True, True)),
         ("GEMM", GemmConfig(128, 128, 32, 64, 32, 5, 4, False, False, True, True, 16, 2)),
+        ("GEMM", GemmConfig(256, 256, 64, 128, 64, 2, 0, True, True, True, False, 16, 4, True)),
         ("GEMM", GemmConfig(256, 128, 64, 128, 64, 1, 1, True, False, False)),
         ("softmax", RowConfig(256, 2, 8, "reg", 1, True)),
         ("rmsnorm", RowConfig(1024, 1, 4, "twopass", 4)),
