@@ -108,11 +108,11 @@ class Tuner:
         return self.tune(*shape, log=log, **kw)
 
     # -- operator specifics -------------------------------------------------------
-    def _make_op(self, shape, dtype="float16", eps=1e-6, causal=False, **_):
+    def _make_op(self, shape, dtype="float16", eps=1e-6, causal=False, inputs="normal", **_):
         from deca_amd import operators as ops
 
         if self.operator == "GEMM":
-            return ops.GEMMTC(*shape, dtype=dtype)
+            return ops.GEMMTC(*shape, dtype=dtype, inputs=inputs)
         if self.operator == "softmax":
             return ops.Softmax(*shape, dtype)
         if self.operator == "rmsnorm":
@@ -288,7 +288,8 @@ class Tuner:
             unit = "GB/s" if self.operator in ("softmax", "rmsnorm") else "TFLOPS"
             tuned.store(key, best_cfg, best, unit, self.cache_path, runtime_ms=round(best_t * 1e3, 4),
                         max_err=float(f"{err_of[best_cfg]:.3e}"), measured_on=self.arch.name,
-                        candidates=len(ranked))
+                        candidates=len(ranked),
+                        **({"inputs": "U(-1,1)"} if getattr(op, "inputs", "normal") == "uniform" else {}))
         for kern in keep:
             kern.close()
         return best_cfg, best, ref

@@ -16,10 +16,14 @@ class GEMMTC(Operator):
     metric = "TFLOPS"
 
     def __init__(self, M: int, N: int, K: int, dtype: str = "float16", acc: str = "fp32",
-                 acc_splits: int = 1, name: str = "GEMMTC"):
+                 acc_splits: int = 1, name: str = "GEMMTC", inputs: str = "normal"):
         """`acc` must be "fp32": the matrix cores of CDNA4 have no fp16
         accumulation, so the reference's acc="fp16" / acc_splits modes
-        (GEMMTC.py:29-43) do not exist here."""
+        (GEMMTC.py:29-43) do not exist here.  `inputs`: "normal" draws N(0, 1)
+        operands as the reference does (gemm_bench.py:29-30), "uniform" U(-1, 1); on a
+        power-limited board the operand statistics decide which tile body is fastest."""
+        assert inputs in ("normal", "uniform")
+        self.inputs = inputs
         from deca_amd.kernels.rowwise_bench import canonical_dtype
 
         dtype = canonical_dtype(dtype)  # "float16" (the reference's only type) or "bfloat16"
@@ -54,7 +58,7 @@ class GEMMTC(Operator):
 
         from deca_amd.kernels.rowwise_bench import torch_dtype
 
-        return make_inputs(self.M, self.N, self.K, dtype=torch_dtype(self.dtype))
+        return make_inputs(self.M, self.N, self.K, dist=self.inputs, dtype=torch_dtype(self.dtype))
 
     def make_output(self, inputs):
         import torch
@@ -75,4 +79,5 @@ class GEMMTC(Operator):
             torch.backends.cuda.matmul.allow_tf32 = saved
 
     def describe(self) -> str:
-        return f"{self.name}(M={self.M}, N={self.N}, K={self.K}, {self.dtype})"
+        dist = ", U(-1,1) inputs" if self.inputs == "uniform" else ""
+        return f"{self.name}(M={self.M}, N={self.N}, K={self.K}, {self.dtype}{dist})"

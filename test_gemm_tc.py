@@ -32,6 +32,8 @@ def parse_args(argv=None):
                         help="tune the square 2K-16K benchmark grid")
     parser.add_argument("--dtype", choices=["fp16", "bf16"], default="fp16",
                         help="type of A, B and C (accumulation is always fp32)")
+    parser.add_argument("--inputs", choices=["normal", "uniform"], default="normal",
+                        help="operand distribution: N(0,1) as the reference, or U(-1,1)")
     parser.add_argument("--top_n", type=int, default=24,
                         help="number of ranked configs to compile and measure (0 = all)")
     parser.add_argument("--jobs", type=int, default=min(16, os.cpu_count() or 1),
@@ -61,7 +63,7 @@ def tune(args, shape, arch, arch_str, log):
 
     tuner = Tuner("GEMM", arch, arch_str, args.top_n, args.jobs, args.finalists, args.rounds,
                   cache_path=_cache_path(args), retune=args.retune)
-    return tuner.tune(*shape, log=log, dtype=args.dtype)
+    return tuner.tune(*shape, log=log, dtype=args.dtype, inputs=args.inputs)
 
 
 def write_sweep_csv(summary, path):
