@@ -138,6 +138,53 @@ def check_generated_code(spec: KernelSpec, asm_text: str) -> None:
             f"{spec.template} [{meta.get('cfg', '')}]: {got} accumulation-register moves where "
             f"{want} are accounted for, {sum(spills)} spilled registers: the compiler moves "
             "accumulators it cannot know to be in flight")
+    late = late_operand_writes(asm_text)
+    if late:
+        raise RuntimeError(
+            f"{spec.template} [{meta.get('cfg', '')}]: accumulation-register moves aside, a vector "
+            f"instruction writes an MFMA operand less than two wait states before it: {late[0]}")
+
+
+def _vgprs(operand: str) -> set:
+    """Vector registers named by one assembly operand: v7, v[4:7]; anything else: none."""
+    m = re.fullmatch(r"v(\d+)", operand)
+    if m:
+        return {int(m.group(1))}
+    m = re.fullmatch(r"v\[(\d+):(\d+)\]", operand)
+    return set(range(int(m.group(1)), int(m.group(2)) + 1)) if m else set()
+
+
+def late_operand_writes(asm_text: str) -> list:
+    """MFMAs with accumulation-register results (the hand-written ones) whose A or B operand
+    is written by a vector-ALU instruction fewer than two wait states earlier, in program
+    text order: every instruction between counts one state, `s_nop n` counts n + 1.  The
+    hardware needs two; the compiler provides them for MFMAs it knows, not behind inline
+    assembly.  Returns descriptions of the offending pairs."""
+    bad, recent = [], []  # recent: (states this instruction adds, registers it writes, text)
+    for raw in asm_text.splitlines():
+        line = raw.split(";")[0].strip()
+        if not line or line.startswith(".") or line.endswith(":"):
+            continue
+        op, _, rest = line.partition(" ")
+        args = [a.strip() for a in rest.split(",")] if rest else []
+        if op.startswith("v_mfma") and args and args[0].startswith("a"):
+            reads = _vgprs(args[1]) | _vgprs(args[2]) if len(args) > 2 else set()
+            states = 0
+            for adds, writes, text in reversed(recent):
+                if states >= 2:
+                    break
+                if writes & reads:
+                    bad.append(f"`{text}` before `{line}`")
+                    break
+                states += adds
+        if op == "s_nop":
+            recent.append((int(args[0]) + 1 if args else 1, set(), line))
+        elif op.startswith("v_") and not op.startswith("v_mfma") and not op.startswith("v_cmp"):
+            recent.append((1, _vgprs(args[0]) if args else set(), line))
+        else:
+            recent.append((1, set(), line))
+        del recent[:-4]
+    return bad
 
 
 def build_kernel(spec: KernelSpec, arch: str | None, path: str, dump_dir: str | None = None) -> str:
