@@ -4,11 +4,12 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-extra]
 
 A step is one launch of the workload's kernel over one batch of synthetic
-input already resident in HBM.  Prints ONE JSON line: the headline workload's
-throughput (`value`), its roofline fraction measured with HIP events on the
-launch stream, the torch-CPU baseline timed on this box's host cores, and --
-unless --no-extra -- the same figures for the other benchmark configurations
-under "results".
+input already resident in HBM.  Prints ONE JSON line, last on standard output:
+the headline workload's throughput (`value`), its roofline fraction measured
+with HIP events on the launch stream, the torch-CPU baseline timed on this
+box's host cores, and -- unless --no-extra -- the same figures for the other
+benchmark configurations in compact form under roofline.all and
+cpu_baseline.all.  The full per-workload records go to --full-out.
 """
 
 from __future__ import annotations
@@ -262,14 +263,15 @@ TARGET_FRAC = {
 
 
 def _compact(res):
-    """What a reader needs to recompute one workload's roofline fraction."""
+    """What a reader needs to recompute one workload's roofline fraction:
+    frac = work / (kernel_us * 1e-6) / (peak * 1e9 or 1e12)."""
     rf = res["roofline"]
     row = {
-        "value": round(res["value"], 2), "unit": res["unit"],
+        "value": round(res["value"], 1), "unit": res["unit"],
         "ms_per_step": round(res["ms_per_step"], 5),
-        "kernel_us": round(rf["kernel_us"], 3),
-        "work": rf.get("algorithmic_bytes", rf.get("algorithmic_flops")),
-        "achieved": round(rf["achieved"], 2), "peak": rf["peak"], "frac": round(rf["frac"], 4),
+        "kernel_us": round(rf["kernel_us"], 2),
+        "work": int(rf.get("algorithmic_bytes", rf.get("algorithmic_flops"))),
+        "achieved": round(rf["achieved"], 1), "peak": rf["peak"], "frac": round(rf["frac"], 4),
         "traffic": rf["traffic"], "kernel_config": res["config"],
     }
     target = TARGET_FRAC.get(res["workload"])
@@ -277,6 +279,63 @@ def _compact(res):
         row["target_frac"] = target
         row["target_met"] = bool(rf["frac"] >= target)
     return row
+
+
+def _compact_cpu(cb):
+    """The CPU baseline of a workload without its description."""
+    return {"value": float("%.4g" % cb["value"]), "unit": cb["unit"], "cores": cb["cores"],
+            "seconds": round(cb["seconds"], 4)}
+
+
+# The record has to fit the tail of standard output a harness keeps of a run.
+MAX_RECORD_BYTES = 8192
+
+
+def build_record(results, steps, warmup):
+    """The one JSON object of a run.  `results[0]` is the headline workload; the
+    others appear in compact form under roofline.all / cpu_baseline.all.  The
+    full per-workload records go to a side file, not into the line."""
+    head = results[0]
+    out = {
+        "metric": head["metric"],
+        "value": head["value"],
+        "unit": head["unit"],
+        "n_gpus": 1,
+        "steps": steps,
+        "warmup": warmup,
+        "ms_per_step": head["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": head["dtype"],
+        "data": "synthetic",
+        "config": {"workload": head["workload"], "kernel_config": head["config"]},
+        "roofline": dict(head["roofline"], all={r["workload"]: _compact(r) for r in results}),
+    }
+    if "cpu_baseline" in head:
+        cb = head["cpu_baseline"]
+        out["cpu_baseline"] = {
+            "value": cb["value"], "unit": cb["unit"], "cores": cb["cores"], "kind": cb["kind"],
+            "sample": cb["sample"], "seconds": cb["seconds"],
+            "all": {r["workload"]: _compact_cpu(r["cpu_baseline"])
+                    for r in results if "cpu_baseline" in r}}
+    gated = {r["workload"]: _compact(r) for r in results if r["workload"] in TARGET_FRAC}
+    out["config"]["targets_met"] = sorted(n for n, c in gated.items() if c["target_met"])
+    out["config"]["targets_missed"] = {n: {"frac": c["frac"], "target": c["target_frac"]}
+                                       for n, c in gated.items() if not c["target_met"]}
+    return out
+
+
+def print_table(results, file):
+    """One line per workload."""
+    print(f"[bench] {'workload':32s} {'value':>10s} {'unit':8s} {'kernel us':>10s} {'frac':>6s} "
+          f"{'target':>6s}  config", file=file)
+    for r in results:
+        c = _compact(r)
+        tgt = f"{c['target_frac']:.2f}" if "target_frac" in c else "  -"
+        print(f"[bench] {r['workload']:32s} {c['value']:10.1f} {c['unit']:8s} {c['kernel_us']:10.2f} "
+              f"{c['frac']:6.3f} {tgt:>6s}  {c['kernel_config']}", file=file)
+    file.flush()
 
 
 def run(wl, steps, warmup, with_cpu=True):
@@ -302,6 +361,8 @@ def main():
                          "--workload instead of its stored winner; implies --no-extra")
     ap.add_argument("--no-extra", action="store_true", help="only the headline workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--full-out", default=os.path.join(ROOT, "gpurun_out", "bench_full.json"),
+                    metavar="PATH", help="file for the full per-workload records ('' for none)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: every workload is a single-device kernel "
@@ -320,54 +381,28 @@ def main():
         op = {"gemm": "GEMM", "fa": "flash_attn"}.get(wl["kind"]) or wl["op"]
         wl["cfg"] = tuned.parse_config(op, args.kernel_config)
         args.no_extra = True
-    head = run(wls[args.workload], args.steps, args.warmup, not args.no_cpu)
-    out = {
-        "metric": head["metric"],
-        "value": head["value"],
-        "unit": head["unit"],
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": head["ms_per_step"],
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": head["dtype"],
-        "data": "synthetic",
-        "config": {"workload": args.workload, "kernel_config": head["config"]},
-        "roofline": head["roofline"],
-    }
-    if "cpu_baseline" in head:
-        out["cpu_baseline"] = head["cpu_baseline"]
-    results = [head]
+    results = [run(wls[args.workload], args.steps, args.warmup, not args.no_cpu)]
     if not args.no_extra:
         # the other benchmark configurations, with fewer steps each so that the
         # default run stays within a few minutes
         k = max(5, min(args.steps, 30))
         results += [run(wl, k, min(args.warmup, 5), not args.no_cpu)
                     for name, wl in wls.items() if name != args.workload]
-        out["results"] = results
-    # Every workload of the run in compact form inside the two objects a reader of
-    # the record is sure to keep, and which of the stated targets were met.
-    out["roofline"] = dict(head["roofline"], all={r["workload"]: _compact(r) for r in results})
-    if "cpu_baseline" in head:
-        out["cpu_baseline"] = dict(
-            head["cpu_baseline"],
-            all={r["workload"]: r["cpu_baseline"] for r in results if "cpu_baseline" in r})
-    gated = {r["workload"]: _compact(r) for r in results if r["workload"] in TARGET_FRAC}
-    out["config"]["targets_met"] = sorted(n for n, c in gated.items() if c["target_met"])
-    out["config"]["targets_missed"] = {n: {"frac": c["frac"], "target": c["target_frac"]}
-                                       for n, c in gated.items() if not c["target_met"]}
-    print(json.dumps(out), flush=True)
-    # one line per workload, last on stderr
-    print(f"[bench] {'workload':32s} {'value':>10s} {'unit':8s} {'kernel us':>10s} {'frac':>6s} "
-          f"{'target':>6s}  config", file=sys.stderr)
-    for r in results:
-        c = _compact(r)
-        tgt = f"{c['target_frac']:.2f}" if "target_frac" in c else "  -"
-        print(f"[bench] {r['workload']:32s} {c['value']:10.1f} {c['unit']:8s} {c['kernel_us']:10.2f} "
-              f"{c['frac']:6.3f} {tgt:>6s}  {c['kernel_config']}", file=sys.stderr)
+    out = build_record(results, args.steps, args.warmup)
+    if args.full_out:
+        try:
+            os.makedirs(os.path.dirname(os.path.abspath(args.full_out)), exist_ok=True)
+            with open(args.full_out, "w") as f:
+                json.dump(dict(out, results=results), f, indent=1)
+        except OSError as e:
+            print(f"[bench] full record not written: {e}", file=sys.stderr)
+    # The table first, the record last: nothing follows the JSON line.
+    print_table(results, sys.stderr)
+    line = json.dumps(out, separators=(",", ":"))
+    if len(line) > MAX_RECORD_BYTES:
+        print(f"[bench] record is {len(line)} bytes (limit {MAX_RECORD_BYTES})", file=sys.stderr)
     sys.stderr.flush()
+    print(line, flush=True)
 
 
 if __name__ == "__main__":
