@@ -393,10 +393,13 @@ FA_DOMAINS = {
     "br": (32, 64, 128, 256),
     "bc": (32, 64, 128),
     "nw": (1, 2, 4, 8),
-    "st": (1, 2),
+    "st": (1, 2, 3),  # as the reference (Solver.py:334); 3 in the plain loop only
     "pipe": (0, 1, 2),
     "mfma": (32, 16),  # 16: v_mfma_f32_16x16x32 tiles (plain and slot loop)
+    "qs": (0, 1),  # Q tile staged in LDS and re-read every KV step (Solver.py:335)
 }
+# `swizzle` stays out of the search (the reference enumerates it, Solver.py:336): linear LDS
+# rows are never faster here, `FAConfig(swizzle=False)` exists for the comparison only.
 
 
 def _fa_constraints(arch, B: int, H: int, S_q: int, S_kv: int, D: int, type_size: int,
@@ -407,7 +410,7 @@ def _fa_constraints(arch, B: int, H: int, S_q: int, S_kv: int, D: int, type_size
     simds = arch.simds_per_cu
 
     def build(o, v):
-        br, bc, nw, st, pipe, mfma = (v[k] for k in FA_DOMAINS)
+        br, bc, nw, st, pipe, mfma, qs = (v[k] for k in FA_DOMAINS)
         c = o.const
         slot_bcs = {m: [b for b in FA_DOMAINS["bc"] if slot_schedule_ok(b, D, m)] or [0]
                     for m in FA_DOMAINS["mfma"]}
@@ -423,9 +426,13 @@ def _fa_constraints(arch, B: int, H: int, S_q: int, S_kv: int, D: int, type_size
             # loads of one tile pair fit the 6-bit vector-memory counter
             o.eq(o.urem(bc * cpr, threads), c(0)),
             o.ule(o.udiv(bc * cpr, threads) * 2, c(63)),
+            # (two tile pairs with the three-deep ring, which only the plain loop has)
+            o.implies(o.eq(st, c(3)), o.all_of(o.eq(pipe, c(0)), o.ule(o.udiv(bc * cpr, threads) * 4, c(63)))),
             o.ule(threads, c(arch.max_threads_per_block)),
-            # LDS: `st` K tiles and `st` V tiles
-            o.ule(st * bc * (2 * D * type_size), c(arch.max_dyn_smem_per_block)),
+            # LDS: `st` K tiles and `st` V tiles, and the Q tile when it is staged
+            # (a wave's Q rows are then loaded as whole 1 KiB runs)
+            o.ule((st * bc * 2 + qs * br) * (D * type_size), c(arch.max_dyn_smem_per_block)),
+            o.implies(o.eq(qs, c(1)), o.eq(o.urem(o.udiv(br, nw) * cpr, c(wave)), c(0))),
             # the software-pipelined loop runs one K tile ahead: two slots, two tiles
             o.implies(o.uge(pipe, c(1)), o.all_of(o.eq(st, c(2)), o.uge(o.udiv(c(S_kv), bc), c(2)))),
             # the slot-interleaved loop issues the S^T chains in pairs of 32-key blocks
@@ -442,7 +449,7 @@ def _fa_constraints(arch, B: int, H: int, S_q: int, S_kv: int, D: int, type_size
         s_one = mq * o.udiv(bc, c(2))
         s_acc = o.ite(o.eq(pipe, c(1)), s_one * 2, o.ite(o.eq(pipe, c(2)), o.udiv(s_one * 7, c(4)), s_one))
         p_h = o.ite(o.eq(pipe, c(2)), o.udiv(mq * o.udiv(bc, c(4)), c(2)), mq * o.udiv(bc, c(4)))
-        q_frag = mq * (D // 16 * 4)
+        q_frag = o.ite(o.eq(qs, c(1)), mq * 8, mq * (D // 16 * 4))
         regs = o_acc + s_acc + p_h + q_frag + 16 + mq * 4 + 40
         regs8 = o.udiv(regs + 7, c(8)) * 8
         waves_per_simd = o.udiv(nw + (simds - 1), c(simds))
@@ -458,7 +465,7 @@ def _fa_constraints(arch, B: int, H: int, S_q: int, S_kv: int, D: int, type_size
 
 
 def solve_flash_attn(arch, B: int, H: int, S_q: int, S_kv: int, D: int, type_size: int = 2,
-                     max_est_regs: int = 512, count: int = 256, backend: str = "auto"):
+                     max_est_regs: int = 512, count: int = 1024, backend: str = "auto"):
     """
     Enumerate FlashAttention forward tile configurations.
     Args:
@@ -480,11 +487,12 @@ def solve_flash_attn(arch, B: int, H: int, S_q: int, S_kv: int, D: int, type_siz
 
     cons = _fa_constraints(arch, B, H, S_q, S_kv, D, type_size, max_est_regs)
     results = []
-    for br, bc, nw, st, pipe, mfma in _enumerate(FA_DOMAINS, cons, count, backend):
-        cfg = FAConfig(Br=br, Bc=bc, num_warps=nw, stages=st, pipe=int(pipe), mfma=mfma)
+    for br, bc, nw, st, pipe, mfma, qs in _enumerate(FA_DOMAINS, cons, count, backend):
+        cfg = FAConfig(Br=br, Bc=bc, num_warps=nw, stages=st, pipe=int(pipe), mfma=mfma,
+                       q_in_smem=bool(qs))
         results.append(cfg)
-        # the plain two-stage loop in its one-copy form, where the unrolled one is expected to
+        # the plain ring loop in its one-copy form, where the unrolled one is expected to
         # run out of registers (it interacts with no other constraint: expanded here)
-        if int(pipe) == 0 and st == 2 and register_fill(cfg, D) >= 0.95:
+        if int(pipe) == 0 and st >= 2 and register_fill(cfg, D) >= 0.95:
             results.append(replace(cfg, roll=True))
     return results

@@ -313,6 +313,9 @@ def fa_score(cfg, arch, shape, causal: bool = False) -> float:
     cus = arch.sm_nums
     t_mma = cus / (arch.peak_mma_sync_flops * 1e9)
     t_lds = (1.0 / wq) / arch.smem_bw_per_sm
+    if getattr(cfg, "q_in_smem", False):
+        # the wave's WQ x D Q rows are read again beside the 2 x Bc x D of K and V
+        t_lds *= 1.0 + wq / (2.0 * cfg.Bc)
     t_l2 = (1.0 / cfg.Br) * cus / (arch.l2_bw * 1e9)
     # vector-ALU time per FLOP: (4 + 4) lane-cycles per score element, 4 * D FLOPs each
     valu_rate = cus * arch.simds_per_cu * 16 * arch.sm_clock_hz  # lane-ops per second
@@ -350,6 +353,8 @@ def fa_score(cfg, arch, shape, causal: bool = False) -> float:
         # the unrolled form of a tile this tight is expected to spill (3-67 registers measured)
         if register_fill(cfg, D) >= 0.95:
             pipe *= 0.965
+    if not getattr(cfg, "swizzle", True):
+        pipe *= 0.5  # linear LDS rows: every fragment read is a multi-way bank conflict
     sync = 1.0 / (1.0 + getattr(arch, "fa_cta_sync_penalty", 0.0) * cfg.num_warps / 4 / wgs)
     # longer KV steps amortise the per-step max / barrier; the slot loop has the row
     # statistics inside the matrix work and pays a little less of it

@@ -8,7 +8,12 @@
 //   DECA_B/H/SQ/SKV/D   problem          DECA_BR   query rows per workgroup
 //   DECA_BC             key/value rows per step
 //   DECA_NW             waves per workgroup (each owns BR / NW query rows)
-//   DECA_STAGES         K/V LDS ring depth (1 or 2)
+//   DECA_STAGES         K/V LDS ring depth (1, 2 or 3; 3 in the plain loop only: tiles are
+//                       requested two steps ahead)
+//   DECA_QSMEM          1: the Q tile is staged in LDS once and its fragments are read
+//                       again from there in every KV step (flash_attn_tir.py:263-281,
+//                       345-348) instead of living in VGPRs for the whole kernel
+//   DECA_SWIZZLE        0: K/V/Q rows lie linearly in LDS (no XOR swizzle)
 //   DECA_CAUSAL         1: key j visible to query i iff j <= i (SQ == SKV)
 //   DECA_SCALE          softmax scale
 //   DECA_PIPE           1: S^T of the next tile is computed before the softmax of
@@ -69,6 +74,12 @@
 #ifndef DECA_ROLL
 #define DECA_ROLL 0  // plain loop with two LDS stages: 1 keeps a single copy of the step
 #endif
+#ifndef DECA_QSMEM
+#define DECA_QSMEM 0
+#endif
+#ifndef DECA_SWIZZLE
+#define DECA_SWIZZLE 1
+#endif
 #ifndef DECA_MIN_WAVES
 #define DECA_MIN_WAVES 1  // waves per SIMD the register allocation must leave room for
 #endif
@@ -109,7 +120,9 @@ constexpr int TILE_CHUNKS = BC * CPR;
 constexpr int TILE_BYTES = TILE_CHUNKS * 16;
 constexpr int KV_IT = TILE_CHUNKS / NT;
 constexpr int NKV = DECA_SKV / BC;
-constexpr int LDS_BYTES = 2 * STAGES * TILE_BYTES;
+constexpr int RING_BYTES = 2 * STAGES * TILE_BYTES;
+constexpr int Q_LDS_OFFSET = RING_BYTES;                 // the Q tile follows the K/V ring
+constexpr int LDS_BYTES = RING_BYTES + (DECA_QSMEM ? BR * D_ * 2 : 0);
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr float NEG_INF = -1e30f;
 constexpr float SL2 = static_cast<float>(DECA_SCALE) * LOG2E;
@@ -119,7 +132,9 @@ static_assert(BR % (32 * NW) == 0, "each wave owns a multiple of 32 query rows")
 static_assert(BC % 32 == 0, "BC must be a multiple of 32");
 static_assert(DECA_SQ % BR == 0 && DECA_SKV % BC == 0, "tiles must divide the sequences");
 static_assert(TILE_CHUNKS % NT == 0, "loader coverage");
-static_assert(STAGES == 1 || STAGES == 2, "K/V ring depth");
+static_assert(STAGES >= 1 && STAGES <= 3, "K/V ring depth");
+static_assert(STAGES < 3 || DECA_PIPE == 0, "three stages: plain loop only");
+static_assert(STAGES < 3 || 4 * KV_IT <= 63, "two tile pairs in flight fit the 6-bit counter");
 static_assert(!DECA_CAUSAL || DECA_SQ == DECA_SKV, "causal needs S_q == S_kv");
 static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
 static_assert(2 * KV_IT <= 63, "vmcnt holds 6 bits");
@@ -158,8 +173,15 @@ typedef __attribute__((address_space(3))) void* lptr;
 constexpr bool ROWS_ALIAS = CPR % 16 == 0;
 constexpr int K_XOR_BITS = ROWS_ALIAS ? 4 : 3;
 constexpr int V_XOR_BITS = ROWS_ALIAS ? 2 : 1;  // of the 64-byte group index (chunk bits 2..)
+#if !DECA_SWIZZLE
+// linear rows: every read of a column of chunks hits the same banks
+constexpr int k_swz(int) { return 0; }
+constexpr int v_swz(int) { return 0; }
+#else
 constexpr int k_swz(int row) { return ROWS_ALIAS ? (row & 15) : ((row >> 1) & 7); }
-#if DECA_MFMA16
+#endif
+#if !DECA_SWIZZLE
+#elif DECA_MFMA16
 // (the two 16-lane blocks of a half-wave read rows r and r + 4 of the same 32-byte column
 // range: bit 2 of r moves them to different halves of the 64-byte group)
 constexpr int v_swz(int row) {
@@ -345,6 +367,23 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
   const int lq = l32;
   const int lg = half;
 #endif
+#if DECA_QSMEM
+  // The wave's WQ rows of Q go to LDS once, in the K tile's layout (chunk c of row r at
+  // slot c ^ k_swz(r)), by the same direct loads as the K/V tiles; the first wait of the
+  // loop covers them.  Only this wave reads them back, so no workgroup barrier is owed.
+  {
+    constexpr int Q_IT = WQ * CPR / 64;
+    static_assert((WQ * CPR) % 64 == 0, "a wave's Q rows are whole 1 KiB runs");
+    const unsigned dst = lds_u + Q_LDS_OFFSET + wave_u * (WQ * D_ * 2);
+    const _Float16* q_origin = Q + (static_cast<size_t>(bh) * DECA_SQ + qt * BR + wave_u * WQ) * D_;
+#pragma unroll
+    for (int it = 0; it < Q_IT; ++it) {
+      const int sidx = it * 64 + lane;
+      const int row = sidx / CPR, cs = sidx % CPR;
+      dma16(q_origin, static_cast<unsigned>(row * D_ + (cs ^ k_swz(row)) * 8) * 2u, dst + it * 1024);
+    }
+  }
+#else
   half8 qf[MQ][DK];
 #pragma unroll
   for (int mq = 0; mq < MQ; ++mq)
@@ -352,6 +391,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
     for (int ks = 0; ks < DK; ++ks)
       qf[mq][ks] = *reinterpret_cast<const half8*>(
           q_base + (mq * TQ + lq) * D_ + ks * (K_CHUNKS_PER_STEP * 8) + lg * 8);
+#endif
 
   acc_t o_acc[DT][MQ];
 #pragma unroll
@@ -378,6 +418,15 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
   auto k_frag_offset = [&](int ks, int kt) __attribute__((always_inline)) {
     return (k_lane_base ^ k_xor_const(ks * K_CHUNKS_PER_STEP)) + k_add_const(ks * K_CHUNKS_PER_STEP) +
            static_cast<unsigned>(kt * TQ * CPR * 16);
+  };
+  // Q fragment (mq, ks): from the registers, or -- the wave's rows lie in LDS like a K tile
+  // whose 32- (16-) row block mq is the query tile -- by the same address as a K fragment.
+  auto q_frag = [&](int mq, int ks) __attribute__((always_inline)) -> half8 {
+#if DECA_QSMEM
+    return *reinterpret_cast<const half8*>(lds + Q_LDS_OFFSET + wave_u * (WQ * D_ * 2) + k_frag_offset(ks, mq));
+#else
+    return qf[mq][ks];
+#endif
   };
   // V: row = kk*16 + r*8 + (half*4 + ti/4), chunk = (dt*4 + tb%2*2 + ti%4/2) ^ v_swz(row)
   // (16x16x32: row = block*16 + (lane/16)*4 + ti/4, chunk = (dt*2 + ti%4/2) ^ v_swz(row))
@@ -408,12 +457,15 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
         for (int e = 0; e < ACC_N; ++e) s_acc[kt][mq][e] = 0.0f;
 #pragma unroll
     for (int ks = 0; ks < DK; ++ks) {
+      half8 qk[MQ];
+#pragma unroll
+      for (int mq = 0; mq < MQ; ++mq) qk[mq] = q_frag(mq, ks);
 #pragma unroll
       for (int kt = 0; kt < KT; ++kt) {
         const half8 kf = *reinterpret_cast<const half8*>(k_lds + k_frag_offset(ks, kt));
 #pragma unroll
         for (int mq = 0; mq < MQ; ++mq)
-          s_acc[kt][mq] = DECA_MFMA(kf, qf[mq][ks], s_acc[kt][mq], 0, 0, 0);
+          s_acc[kt][mq] = DECA_MFMA(kf, qk[mq], s_acc[kt][mq], 0, 0, 0);
       }
     }
   };
@@ -549,12 +601,30 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
     DECA_WAIT_VMCNT(0);                  // this lane's outstanding tile loads have landed
     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wave's LDS reads have returned
     __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");       // no LDS read of the new tile moves above the barrier
   };
 
-#if STAGES == 2
-  // One KV step.  `slot` is a literal at both call sites, so that every LDS
-  // address of the step is "lane base + immediate" and needs no address arithmetic.
+#if STAGES >= 2
+  // One KV step.  `slot` is a literal at the call sites of the unrolled loops, so that
+  // every LDS address of the step is "lane base + immediate" and needs no address arithmetic.
   auto kv_step = [&](int j, int slot) __attribute__((always_inline)) {
+#if STAGES == 3
+    // Tiles are requested two steps ahead.  Loads return in order, so tile j has landed
+    // for this lane once only the pair of tile j+1 is still outstanding; after the
+    // barrier every wave is done with the slot of tile j-1, which tile j+2 takes.
+    if (j + 1 < nkv)
+      DECA_WAIT_VMCNT(2 * KV_IT);
+    else
+      DECA_WAIT_VMCNT(0);
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    if (j + 2 < nkv) {
+      const int fill = slot == 0 ? 2 : slot - 1;
+      issue_k(j + 2, fill);
+      issue_v(j + 2, fill);
+    }
+#else
     // Tile j has landed for every lane, and every wave is done with the slot
     // that tile j+1 is about to overwrite.
     wait_and_barrier();
@@ -562,6 +632,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
       issue_k(j + 1, slot ^ 1);
       issue_v(j + 1, slot ^ 1);
     }
+#endif
 #if DECA_CAUSAL
     // Every key of the tile lies after every query row of this wave (the last tile
     // of a workgroup with BR > BC): all its scores are masked, P = 0 exactly, and
@@ -672,7 +743,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
 #pragma unroll
       for (int mq = 0; mq < MQ; ++mq)
         s_nxt[kt][mq] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
-            kf, qf[mq][ks], ks == 0 ? zero : s_nxt[kt][mq], 0, 0, 0);
+            kf, q_frag(mq, ks), ks == 0 ? zero : s_nxt[kt][mq], 0, 0, 0);
 #pragma unroll
       for (int mq = 0; mq < MQ; ++mq)
 #pragma unroll
@@ -829,7 +900,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
         constexpr int pr = t / (2 * DK), r = t % (2 * DK), ks = r / 2, kt = 2 * pr + r % 2;
         static_for<MQ>([&](auto mqc) {
           constexpr int mq = decltype(mqc)::value;
-          sn[kt][mq] = DECA_MFMA(frag[t % 3], qf[mq][ks], ks == 0 ? zero : sn[kt][mq], 0, 0, 0);
+          sn[kt][mq] = DECA_MFMA(frag[t % 3], q_frag(mq, ks), ks == 0 ? zero : sn[kt][mq], 0, 0, 0);
         });
       } else {
         constexpr int u = t - S_SLOTS, kk = u / DT, dt = u % DT;
@@ -972,7 +1043,22 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
 #else
   issue_k(0, 0);
   issue_v(0, 0);
-#if STAGES == 2 && DECA_ROLL
+#if STAGES == 3
+  if (nkv > 1) {
+    issue_k(1, 1);
+    issue_v(1, 1);
+  }
+#if DECA_ROLL
+#pragma unroll 1
+  for (int j = 0, slot = 0; j < nkv; ++j, slot = slot == 2 ? 0 : slot + 1) kv_step(j, slot);
+#else
+  for (int j = 0; j < nkv; j += 3) {
+    kv_step(j, 0);
+    if (j + 1 < nkv) kv_step(j + 1, 1);
+    if (j + 2 < nkv) kv_step(j + 2, 2);
+  }
+#endif
+#elif STAGES == 2 && DECA_ROLL
   // one copy of the step, the ring slot a run-time value
 #pragma unroll 1
   for (int j = 0; j < nkv; ++j) kv_step(j, j & 1);

@@ -11,9 +11,13 @@ What changes on CDNA4: a wave is 64 lanes and owns a multiple of 32 query rows
 products are computed transposed (S^T = K Q^T, O^T = V^T P^T) so that P stays in
 registers between them -- the MFMA accumulator layout is not the operand layout,
 unlike mma.sync m16n8k16 (:8-9); K/V tiles arrive by asynchronous global->LDS
-loads (cp.async, :320-335); Q is read from global memory straight into VGPRs, so
-there is no Q tile in LDS and `q_in_smem` is not offered; the LDS layout is
-always swizzled.
+loads (cp.async, :320-335).  Q is read from global memory straight into VGPRs and
+stays there; with `q_in_smem` the Q tile is staged in LDS behind the K/V ring once
+and each wave reads its fragments again in every KV step (:263-281, :345-348),
+which trades `D/4` registers per query tile for LDS reads.  `swizzle=False` keeps
+the LDS rows linear: the direct loads write whole 1 KiB runs, so rows cannot be
+padded as the reference does (:105) and the unswizzled form is only the slow
+baseline of the comparison.
 """
 
 from __future__ import annotations
@@ -37,9 +41,9 @@ class FAConfig:
     Br: int = 128  # Q rows per workgroup
     Bc: int = 64  # KV rows per pipeline step
     num_warps: int = 4
-    stages: int = 2  # K/V LDS ring depth
-    q_in_smem: bool = False  # kept for the record format; Q always lives in VGPRs here
-    swizzle: bool = True  # kept for the record format; the LDS layout is always swizzled
+    stages: int = 2  # K/V LDS ring depth (1..3; 3 requests tiles two steps ahead, plain loop)
+    q_in_smem: bool = False  # re-read Q fragments from LDS every KV step (else VGPR resident)
+    swizzle: bool = True  # XOR swizzle of the LDS rows (else linear rows, bank conflicts)
     # 0: S^T, softmax, O^T of one tile after the other.  1: S^T of tile j+1 is computed
     # before the softmax of tile j (two S^T accumulators).  2: as 1, and every matrix
     # instruction of an iteration carries a fixed share of its vector work.
@@ -70,8 +74,9 @@ class FAConfig:
 
 
 def smem_bytes(cfg: FAConfig, D: int) -> int:
-    """`stages` K tiles and `stages` V tiles of Bc x D halves (no Q tile)."""
-    return 2 * cfg.stages * cfg.Bc * D * 2
+    """`stages` K tiles and `stages` V tiles of Bc x D halves, and the Q tile when it is
+    staged (flash_attn_tir.py:54-56; rows are never padded here)."""
+    return (2 * cfg.stages * cfg.Bc + (cfg.Br if cfg.q_in_smem else 0)) * D * 2
 
 
 def est_regs_per_thread(cfg: FAConfig, D: int) -> int:
@@ -85,7 +90,8 @@ def est_regs_per_thread(cfg: FAConfig, D: int) -> int:
     elif int(cfg.pipe) == 2:
         # tile j's scores turn into packed halves while tile j+1's chains come to life
         s_acc, p_h = s_acc * 7 // 4, p_h // 2
-    q_frag = mq * (D // 16) * 4
+    # Q fragments: all of them, or two k-steps' worth in flight (flash_attn_tir.py:65)
+    q_frag = 2 * mq * 4 if cfg.q_in_smem else mq * (D // 16) * 4
     kv_frag = 2 * 4 * 2  # a few K / V fragments in flight
     return o_acc + s_acc + p_h + q_frag + kv_frag + 4 * mq + 40
 
@@ -96,7 +102,7 @@ def est_regs_per_thread(cfg: FAConfig, D: int) -> int:
 # estimate for the plain loop with one LDS stage, 1.5x and more with two (the two unrolled
 # steps overlap), 1.0-1.3x for the loops whose order is fixed by hand.  Beyond these the
 # kernels spill to scratch memory inside the loop and run 2-15x slower.
-SPILL_FREE_EST_REGS = {(0, 1): 365, (0, 2): 330, (1, 2): 480, (2, 2): 480}
+SPILL_FREE_EST_REGS = {(0, 1): 365, (0, 2): 330, (0, 3): 330, (1, 2): 480, (2, 2): 480}
 
 
 def expect_spill_free(cfg: FAConfig, D: int) -> bool:
@@ -161,14 +167,17 @@ def check_config(cfg: FAConfig, S_q: int, S_kv: int, D: int) -> None:
     assert (cfg.Bc * cpr) % cfg.threads == 0
     assert 2 * (cfg.Bc * cpr) // cfg.threads <= 63
     assert cfg.threads <= 1024
-    assert cfg.stages in (1, 2)
+    assert cfg.stages in (1, 2, 3)
+    assert cfg.stages < 3 or int(cfg.pipe) == 0, "three stages: plain loop only"
+    assert cfg.stages < 3 or 4 * (cfg.Bc * cpr) // cfg.threads <= 63
     assert int(cfg.pipe) in (0, 1, 2)
     assert cfg.mfma in (32, 16)
     assert cfg.mfma == 32 or int(cfg.pipe) != 1, "the 16x16x32 form exists for the plain and the slot loop"
     assert not cfg.pipe or cfg.stages == 2
-    assert not cfg.roll or (int(cfg.pipe) == 0 and cfg.stages == 2), "roll is a form of the plain two-stage loop"
+    assert not cfg.roll or (int(cfg.pipe) == 0 and cfg.stages >= 2), "roll is a form of the plain ring loop"
     assert int(cfg.pipe) != 2 or slot_schedule_ok(cfg.Bc, D, cfg.mfma)
-    assert not cfg.q_in_smem and cfg.swizzle
+    # a wave's Q rows go to LDS as whole 1 KiB runs
+    assert not cfg.q_in_smem or (cfg.Br // cfg.num_warps * cpr) % WAVE == 0
     assert smem_bytes(cfg, D) <= MAX_LDS
     assert est_regs_per_thread(cfg, D) <= 512
 
@@ -202,9 +211,17 @@ def make_flash_attn_fwd(
         defines["DECA_MFMA16"] = 1
     if cfg.roll:
         defines["DECA_ROLL"] = 1
+    if cfg.q_in_smem:
+        defines["DECA_QSMEM"] = 1
+    if not cfg.swizzle:
+        defines["DECA_SWIZZLE"] = 0
+    # The three-stage ring waits for part of its outstanding loads, which is only right
+    # while the tile loads are the loop's only vector-memory traffic: a build that spills
+    # (scratch stores share the counter and retire out of order) is refused at load time.
     return make_spec(
         TEMPLATE, defines, grid=((S_q // cfg.Br) * B * H, 1, 1), block=(cfg.threads, 1, 1), nargs=4,
-        options=FAST_MATH_OPTIONS, meta={"cfg": str(cfg), "causal": causal},
+        options=FAST_MATH_OPTIONS,
+        meta={"cfg": str(cfg), "causal": causal, "no_scratch": cfg.stages > 2},
     )
 
 

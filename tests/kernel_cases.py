@@ -208,6 +208,36 @@ FA_CASES = [
     (1, 2, 512, 512, 128, True, FAConfig(256, 128, 8, 2, roll=True)),
     (2, 2, 256, 320, 64, False, FAConfig(128, 64, 4, 2, roll=True)),
     (1, 2, 512, 512, 64, True, FAConfig(128, 64, 4, 2, mfma=16, roll=True)),
+    # Q tile staged in LDS, its fragments read again in every KV step: full and causal,
+    # D = 64 / 128 / 192, both tile forms, one to three LDS stages, the three loops, rolled
+    (1, 2, 512, 512, 128, False, FAConfig(256, 64, 8, 2, q_in_smem=True)),
+    (1, 2, 512, 512, 128, True, FAConfig(256, 64, 8, 2, q_in_smem=True, mfma=16)),
+    (2, 2, 512, 512, 64, False, FAConfig(256, 128, 4, 2, q_in_smem=True, mfma=16)),
+    (2, 2, 512, 512, 64, True, FAConfig(128, 64, 4, 2, q_in_smem=True)),
+    (1, 2, 256, 256, 192, False, FAConfig(128, 32, 4, 2, q_in_smem=True, mfma=16)),
+    (1, 2, 256, 256, 192, True, FAConfig(64, 64, 2, 1, q_in_smem=True)),
+    (1, 3, 128, 640, 128, False, FAConfig(64, 64, 2, 1, q_in_smem=True, mfma=16)),
+    (1, 2, 512, 512, 128, True, FAConfig(256, 64, 8, 2, q_in_smem=True, pipe=1)),
+    (1, 2, 512, 512, 128, False, FAConfig(256, 64, 8, 2, q_in_smem=True, pipe=2)),
+    (2, 2, 512, 512, 64, True, FAConfig(256, 128, 8, 2, q_in_smem=True, pipe=2, mfma=16)),
+    (1, 2, 512, 512, 128, True, FAConfig(128, 128, 4, 2, q_in_smem=True, mfma=16, roll=True)),
+    (1, 2, 512, 512, 64, False, FAConfig(256, 64, 4, 3, q_in_smem=True, roll=True)),
+    # three LDS stages (tiles requested two steps ahead): 1, 2, 4, 5 and 8 KV tiles, full and
+    # causal, both tile forms, unrolled by three and rolled
+    (1, 2, 128, 64, 64, False, FAConfig(64, 64, 2, 3)),
+    (1, 2, 128, 128, 128, True, FAConfig(64, 64, 2, 3, mfma=16)),
+    (1, 2, 256, 256, 128, False, FAConfig(128, 64, 4, 3)),
+    (1, 2, 256, 320, 64, False, FAConfig(128, 64, 2, 3, mfma=16)),
+    (1, 2, 512, 512, 128, True, FAConfig(128, 64, 4, 3)),
+    (2, 2, 512, 512, 64, True, FAConfig(256, 64, 4, 3, mfma=16, roll=True)),
+    (1, 2, 256, 320, 128, False, FAConfig(128, 64, 4, 3, roll=True)),
+    (1, 2, 512, 512, 192, True, FAConfig(128, 32, 4, 3, q_in_smem=True, mfma=16)),
+    # linear LDS rows (no swizzle): both row lengths, both tile forms, with and without the
+    # staged Q tile
+    (1, 2, 256, 256, 128, True, FAConfig(128, 64, 4, 2, swizzle=False)),
+    (1, 2, 256, 256, 64, False, FAConfig(128, 64, 4, 2, swizzle=False, mfma=16)),
+    (1, 2, 256, 256, 64, True, FAConfig(128, 64, 4, 1, q_in_smem=True, swizzle=False)),
+    (1, 2, 512, 512, 128, False, FAConfig(256, 64, 8, 2, q_in_smem=True, swizzle=False, pipe=2, mfma=16)),
 ]
 
 FA_FULL = [
@@ -219,6 +249,8 @@ FA_FULL = [
     (4, 16, 4096, 4096, 64, False, FAConfig(256, 128, 8, 2, pipe=2)),
     (4, 16, 4096, 4096, 128, False, FAConfig(256, 64, 8, 2, pipe=2)),
     (4, 16, 4096, 4096, 128, True, FAConfig(256, 64, 8, 2, pipe=2)),
+    (4, 16, 4096, 4096, 128, False, FAConfig(256, 64, 8, 2, q_in_smem=True, mfma=16)),
+    (4, 16, 4096, 4096, 64, True, FAConfig(256, 64, 4, 3, q_in_smem=True)),
 ]
 
 

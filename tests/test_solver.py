@@ -141,9 +141,9 @@ def test_flash_attn_configs_are_valid(D, S):
         fa.check_config(cfg, S, S, D)
         assert (S // cfg.Br) * B * H >= ARCH.sm_nums
     want = set()
-    for br, bc, nw, st, pipe, mfma in itertools.product(
-            (32, 64, 128, 256), (32, 64, 128), (1, 2, 4, 8), (1, 2), (0, 1, 2), (32, 16)):
-        cfg = fa.FAConfig(br, bc, nw, st, pipe=pipe, mfma=mfma)
+    for br, bc, nw, st, pipe, mfma, qs in itertools.product(
+            (32, 64, 128, 256), (32, 64, 128), (1, 2, 4, 8), (1, 2, 3), (0, 1, 2), (32, 16), (0, 1)):
+        cfg = fa.FAConfig(br, bc, nw, st, pipe=pipe, mfma=mfma, q_in_smem=bool(qs))
         try:
             fa.check_config(cfg, S, S, D)
         except AssertionError:
@@ -154,10 +154,14 @@ def test_flash_attn_configs_are_valid(D, S):
         if regs * -(-nw // 4) > 512 or not fa.expect_spill_free(cfg, D):
             continue
         want.add(cfg)
-        # the one-copy form of the plain two-stage loop, where the unrolled one is tight
-        if pipe == 0 and st == 2 and fa.register_fill(cfg, D) >= 0.95:
+        # the one-copy form of the plain ring loop, where the unrolled one is tight
+        if pipe == 0 and st >= 2 and fa.register_fill(cfg, D) >= 0.95:
             want.add(replace(cfg, roll=True))
     assert set(configs) == want
+    # the reference's knobs are all in the search (Solver.py:330-336), except linear LDS rows
+    assert {c.stages for c in configs} == {1, 2, 3}
+    assert {c.q_in_smem for c in configs} == {False, True} and all(c.swizzle for c in configs)
+    assert all(fa.smem_bytes(c, D) <= ARCH.max_dyn_smem_per_block for c in configs)
     # a tighter register budget removes the widest per-wave tiles
     tight = Solver.solve_flash_attn(ARCH, B, H, S, S, D, max_est_regs=256)
     assert set(tight) < set(configs) or set(tight) == set(configs)
@@ -247,6 +251,33 @@ def test_flash_attn_rolled_loop_is_offered_where_registers_are_tight():
     assert dict(fa.make_flash_attn_fwd(4, 16, 4096, 4096, 128, next(iter(rolled))).defines)["DECA_ROLL"] == 1
     with pytest.raises(AssertionError):
         fa.check_config(fa.FAConfig(256, 64, 8, 2, pipe=2, roll=True), 4096, 4096, 128)
+
+
+def test_flash_attn_knobs_of_the_reference():
+    """`q_in_smem`, `swizzle` and `stages` 1..3 (flash_attn_tir.py:35-38) all reach the
+    kernel: LDS footprint, register estimate and the macros of the specialisation."""
+    base = fa.FAConfig(256, 64, 8, 2)
+    staged = replace(base, q_in_smem=True)
+    assert fa.smem_bytes(base, 128) == 2 * 2 * 64 * 128 * 2
+    assert fa.smem_bytes(staged, 128) == fa.smem_bytes(base, 128) + 256 * 128 * 2
+    # all D/16 fragments of a query tile against two in flight (flash_attn_tir.py:65)
+    assert fa.est_regs_per_thread(base, 128) - fa.est_regs_per_thread(staged, 128) == (128 // 16 - 2) * 4
+    defs = dict(fa.make_flash_attn_fwd(4, 16, 4096, 4096, 128, staged).defines)
+    assert defs["DECA_QSMEM"] == 1 and "DECA_SWIZZLE" not in defs
+    defs = dict(fa.make_flash_attn_fwd(4, 16, 4096, 4096, 128, replace(base, swizzle=False)).defines)
+    assert defs["DECA_SWIZZLE"] == 0 and "DECA_QSMEM" not in defs
+    deep = fa.FAConfig(128, 64, 4, 3)
+    spec = fa.make_flash_attn_fwd(4, 16, 4096, 4096, 128, deep)
+    assert dict(spec.defines)["DECA_STAGES"] == 3 and dict(spec.meta)["no_scratch"] is True
+    assert dict(fa.make_flash_attn_fwd(4, 16, 4096, 4096, 128, base).meta)["no_scratch"] is False
+    assert str(staged).find("q_smem=1") > 0 and str(replace(base, swizzle=False)).find("swz=0") > 0
+    # the winner tile of D = 128 (a 128 KiB ring) has no room for a 64 KiB Q tile
+    with pytest.raises(AssertionError):
+        fa.check_config(fa.FAConfig(256, 128, 8, 2, q_in_smem=True), 4096, 4096, 128)
+    # three stages belong to the plain loop; four do not exist
+    for bad in (fa.FAConfig(128, 64, 4, 3, pipe=2), fa.FAConfig(128, 64, 4, 3, pipe=1), fa.FAConfig(128, 64, 4, 4)):
+        with pytest.raises(AssertionError):
+            fa.check_config(bad, 4096, 4096, 128)
 
 
 def test_flash_attn_head_dims():
