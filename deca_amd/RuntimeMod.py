@@ -21,14 +21,22 @@ _VERIFY_ELEMS = 1 << 24
 
 
 class RuntimeMod:
-    def __init__(self, operator: Operator, arch, use_tc: bool, compute_pattern):
+    def __init__(self, operator: Operator, arch, use_tc: bool, compute_pattern,
+                 timing: str = "events"):
         """
         Args:
             operator: the operator whose kernel is tuned
             arch: hardware model of the GPU
             use_tc: kept for signature compatibility (every GEMM here uses MFMA)
             compute_pattern: the config (`GemmConfig`, `RowConfig` or `FAConfig`)
+            timing: "events" -- one event pair and one synchronisation per call, the
+                reference's procedure (attn_bench.py:35-70); "back_to_back" -- batches of
+                launches between one event pair (`deca_launch_timed`)
         """
+        from deca_amd.kernels.attn_bench import TIMINGS
+
+        assert timing in TIMINGS, timing
+        self.timing = timing
         self.operator = operator
         self.arch = arch
         self.use_tc = use_tc
@@ -105,7 +113,7 @@ class RuntimeMod:
         `abs_tol`: absolute tolerance (attention); None: the operator's (atol, rtol)."""
         import torch
 
-        from deca_amd.kernels.attn_bench import bench_cuda
+        from deca_amd.kernels.attn_bench import bench_back_to_back, bench_cuda
 
         if self.runtime_mod is None:
             raise RuntimeError("no kernel loaded: call build() or load_kernel(path) first")
@@ -134,9 +142,15 @@ class RuntimeMod:
             from deca_amd.kernels.rowwise_bench import cycle, rotating_sets
 
             sets = rotating_sets(inputs, args[-1], getattr(self.arch, "mall_bytes", 0))
-            self.execution_time = t = bench_cuda(cycle(kern, sets))
+            if self.timing == "back_to_back":
+                t = bench_back_to_back(lambda n: kern.time(sets, n))
+            else:
+                t = bench_cuda(cycle(kern, sets))
+        elif self.timing == "back_to_back":
+            t = bench_back_to_back(lambda n: kern.time([args], n))
         else:
-            self.execution_time = t = bench_cuda(lambda: kern(*args))
+            t = bench_cuda(lambda: kern(*args))
+        self.execution_time = t
         return t
 
     # ---- timing ----------------------------------------------------------------------------

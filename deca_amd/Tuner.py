@@ -77,8 +77,16 @@ class Tuner:
 
     def __init__(self, operator: str = "GEMM", arch=None, arch_str: str | None = None,
                  top_n: int | None = None, jobs: int | None = None, finalists: int = 3,
-                 rounds: int = 5, cache_path: str | None = None, retune: bool = False):
+                 rounds: int = 5, cache_path: str | None = None, retune: bool = False,
+                 timing: str = "back_to_back"):
+        from deca_amd.kernels.attn_bench import TIMINGS
+
         assert operator in self.OPERATORS
+        assert timing in TIMINGS, timing
+        # "back_to_back": candidates and finalists are timed in batches of launches between
+        # one event pair, as bench.py times them; "events": one event pair and one
+        # synchronisation per call, the reference's procedure (attn_bench.py:35-70)
+        self.timing = timing
         self.operator = operator
         if arch is None:
             from deca_amd.utils.helper import GPUDetector
@@ -199,7 +207,9 @@ class Tuner:
         """Returns (best config, its throughput, torch's throughput)."""
         import torch
 
-        from deca_amd.kernels.attn_bench import bench_interleaved
+        from deca_amd.kernels.attn_bench import (
+            batch_timer, bench_interleaved, bench_interleaved_batches,
+        )
         from deca_amd.RuntimeMod import RuntimeMod
 
         from deca_amd import tuned
@@ -207,7 +217,7 @@ class Tuner:
         start = time.time()
         op = self._make_op(shape, **kw)
         key = tuned.make_key(self.operator, getattr(op, "shape", shape), op.dtype, self.arch_str,
-                             bool(getattr(op, "causal", False)))
+                             bool(getattr(op, "causal", False)), getattr(op, "inputs", "normal"))
         cached = tuned.lookup(key, self.cache_path) if self.cache_path and not self.retune else None
         if cached is not None and op.is_valid(cached):
             # a stored winner: verify and time it alone instead of searching
@@ -226,7 +236,7 @@ class Tuner:
         for cfg in ranked:
             if cfg not in paths:
                 continue
-            rt = RuntimeMod(op, self.arch, True, cfg)
+            rt = RuntimeMod(op, self.arch, True, cfg, timing=self.timing)
             try:
                 rt.load_kernel(paths[cfg])
                 rt.time_evaluator()
@@ -256,6 +266,7 @@ class Tuner:
         out = op.make_output(inputs) if hasattr(op, "make_output") else torch.empty_like(inputs[0])
         args = op.kernel_args(inputs, out)
         keep = []
+        b2b = self.timing == "back_to_back"
         if self.operator in ("softmax", "rmsnorm"):
             # memory-bound: DeCA and torch both cycle through buffer sets larger
             # than the Infinity Cache, so that both stream from HBM
@@ -266,14 +277,19 @@ class Tuner:
             for _, cfg, _, _ in finalists:
                 kern = load_kernel(op.build_mod(cfg), paths[cfg])
                 keep.append(kern)
-                fns[cfg] = cycle(kern, sets)
+                fns[cfg] = (lambda n, kern=kern: kern.time(sets, n)) if b2b else cycle(kern, sets)
         else:
             fns = {"torch": self._torch_fn(op, inputs)}
             for _, cfg, _, _ in finalists:
                 kern = load_kernel(op.build_mod(cfg), paths[cfg])
                 keep.append(kern)
-                fns[cfg] = lambda kern=kern: kern(*args)
-        times = bench_interleaved(fns, rounds=self.rounds)
+                fns[cfg] = ((lambda n, kern=kern: kern.time([args], n)) if b2b
+                            else (lambda kern=kern: kern(*args)))
+        if b2b:
+            fns["torch"] = batch_timer(fns["torch"])
+            times = bench_interleaved_batches(fns, rounds=self.rounds)
+        else:
+            times = bench_interleaved(fns, rounds=self.rounds)
         torch_t = times.pop("torch")
         best_cfg, best_t = min(times.items(), key=lambda x: x[1])
         msg, best, ref = self._report(
@@ -288,7 +304,11 @@ class Tuner:
             unit = "GB/s" if self.operator in ("softmax", "rmsnorm") else "TFLOPS"
             tuned.store(key, best_cfg, best, unit, self.cache_path, runtime_ms=round(best_t * 1e3, 4),
                         max_err=float(f"{err_of[best_cfg]:.3e}"), measured_on=self.arch.name,
-                        candidates=len(ranked),
+                        # provenance: this search measured `candidates` configs of the
+                        # solver's `solutions`, and the winner was the cost model's `rank`-th
+                        method="tuner", timing=self.timing, candidates=len(ranked),
+                        solutions=len(configs), rank=ranked.index(best_cfg) + 1,
+                        torch_throughput=round(float(ref), 2),
                         **({"inputs": "U(-1,1)"} if getattr(op, "inputs", "normal") == "uniform" else {}))
         for kern in keep:
             kern.close()

@@ -105,6 +105,8 @@ deca_main(const float* __restrict__ in, float* __restrict__ out) {
                      : "+v"(x[4 * i]), "+v"(x[4 * i + 1]), "+v"(x[4 * i + 2]), "+v"(x[4 * i + 3])
                      : "v"(c0), "v"(c1));
 #if DECA_OP == 9 && DECA_ACC_AGPR
+      // (timing probe only: the accumulator read here was written two MFMAs earlier, with
+      // no wait states placed by hand -- what it reads is not used as a value)
       asm volatile("v_accvgpr_read_b32 %0, %2\n\tv_accvgpr_read_b32 %1, %3"
                    : "=v"(x[(4 * i + 5) % 16]), "=v"(x[(4 * i + 6) % 16]) : "a"(acc[(i + 2) % 4][0]), "a"(acc[(i + 2) % 4][1]));
 #endif
@@ -120,6 +122,13 @@ deca_main(const float* __restrict__ in, float* __restrict__ out) {
 #pragma unroll
   for (int i = 0; i < 16; ++i) s += x[i];
 #if DECA_OP >= 4
+#if DECA_ACC_AGPR
+  // The MFMAs above are inline assembly: the compiler places no wait states between the
+  // last of them and the reads of their results below (18 are owed after a 16-pass MFMA).
+  __builtin_amdgcn_sched_barrier(0);
+  asm volatile("s_nop 15\n\ts_nop 3" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);
+#endif
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll

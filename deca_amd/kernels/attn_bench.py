@@ -112,6 +112,54 @@ def bench_interleaved(fns: dict, rounds: int = 3) -> dict:
     return {name: _median(seen) for name, seen in per_name.items()}
 
 
+TIMINGS = ("events", "back_to_back")
+
+
+def batch_timer(fn):
+    """`timed(n)` -> average seconds of n back-to-back calls of `fn` on torch's current
+    stream, between one pair of events.  A kernel loaded by this package brings its own
+    (`LoadedKernel.time`, whose launches stay inside the launcher library); this is for
+    callables that go through torch."""
+    import torch
+
+    first, last = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+    def timed(n: int) -> float:
+        first.record()
+        for _ in range(n):
+            fn()
+        last.record()
+        last.synchronize()
+        return first.elapsed_time(last) * 1e-3 / n
+
+    return timed
+
+
+def bench_back_to_back(timed, warmup_s: float = 0.3, measure_s: float = 0.3,
+                       min_iters: int = 20, batches: int = 3) -> float:
+    """Seconds per call from batches of calls issued back to back (`timed(n)`, see
+    `batch_timer`): a time-based warm-up as in `bench_cuda`, then `batches` batches that
+    together last about `measure_s`; the median batch.  Unlike the one-call-per-event-pair
+    timing of `bench_cuda` (the reference's, attn_bench.py:35-70) the GPU never idles
+    between calls, which is how a kernel runs inside a model and what bench.py times: on a
+    power-limited board the two rank near-equal candidates differently."""
+    deadline = time.perf_counter() + warmup_s
+    settled = timed(4)
+    while time.perf_counter() < deadline:
+        settled = timed(8)
+    count = max(int(min_iters), int(measure_s / max(settled, 1e-7) / batches))
+    return _median([timed(count) for _ in range(batches)])
+
+
+def bench_interleaved_batches(timers: dict, rounds: int = 3) -> dict:
+    """`bench_interleaved` for batch timers (name -> `timed(n)`)."""
+    per_name = {name: [] for name in timers}
+    for _ in range(rounds):
+        for name in per_name:
+            per_name[name].append(bench_back_to_back(timers[name]))
+    return {name: _median(seen) for name, seen in per_name.items()}
+
+
 def make_qkv(B: int, H: int, S_q: int, S_kv: int, D: int, dtype=None, seed: int = 0,
              device: str = "cuda"):
     """q, k, v ~ N(0, 1) in [B, H, S, D] (reference: attn_bench.py:73-78)."""

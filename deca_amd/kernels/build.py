@@ -187,42 +187,76 @@ def late_operand_writes(asm_text: str) -> list:
     return bad
 
 
+# The checks of `check_generated_code` read compiler output as text: which instructions the
+# register allocator adds and where the scheduler puts them is a property of one compiler.
+# They were validated (every `agpr=1` configuration of two shapes built, checked and run
+# against torch on the GPU) with this hipcc; under another one a kernel that relies on them
+# is refused unless DECA_ALLOW_UNCHECKED_HIPCC=1.
+VALIDATED_HIPCC = "HIP version: 7.2.26015"
+_hipcc_version = None
+
+
+def hipcc_version() -> str:
+    """First line of `hipcc --version` (cached)."""
+    global _hipcc_version
+    if _hipcc_version is None:
+        proc = subprocess.run([hipcc_path(), "--version"], capture_output=True, text=True)
+        _hipcc_version = (proc.stdout.splitlines() or [""])[0].strip()
+    return _hipcc_version
+
+
+def require_validated_hipcc(spec: KernelSpec) -> None:
+    if os.environ.get("DECA_ALLOW_UNCHECKED_HIPCC") == "1":
+        return
+    have = hipcc_version()
+    if not have.startswith(VALIDATED_HIPCC):
+        raise RuntimeError(
+            f"{spec.template} [{dict(spec.meta).get('cfg', '')}] relies on checks of the generated "
+            f"code that were validated with '{VALIDATED_HIPCC}...'; this is '{have}'. Set "
+            "DECA_ALLOW_UNCHECKED_HIPCC=1 to build it anyway.")
+
+
 def build_kernel(spec: KernelSpec, arch: str | None, path: str, dump_dir: str | None = None) -> str:
     """Compiles `spec` into the code object `path`; `dump_dir` keeps the
-    generated ISA (`*.s`) for inspection (reference: build.py:73-87).  A spec that makes
-    promises about its generated code (`check_generated_code`) is compiled with the ISA
-    kept and refused when they do not hold."""
+    generated ISA for inspection, as `<template>_<key>.s` (reference: build.py:73-87).  A
+    spec that makes promises about its generated code (`check_generated_code`) is compiled
+    with the ISA kept and refused when they do not hold.  The compiler's intermediate
+    files go to a directory of this build's own, so that neither another build's
+    assembly nor a stale file can be the one that is checked or kept."""
     arch = arch or DEFAULT_ARCH
     os.makedirs(os.path.dirname(os.path.abspath(path)) or ".", exist_ok=True)
     tmp = f"{path}.tmp{os.getpid()}_{threading.get_ident()}"
     cmd = compile_command(spec, arch, tmp)
-    cwd, scratch_dir = None, None
     checked = "accumulator_moves" in dict(spec.meta)
-    if dump_dir:
-        os.makedirs(dump_dir, exist_ok=True)
-        cwd = dump_dir
-    elif checked:
-        scratch_dir = tempfile.mkdtemp(prefix="deca_isa_")
-        cwd = scratch_dir
-    if cwd:
+    if checked:
+        require_validated_hipcc(spec)
+    work_dir = tempfile.mkdtemp(prefix="deca_isa_") if (checked or dump_dir) else None
+    if work_dir:
         cmd.append("--save-temps")
     try:
-        proc = subprocess.run(cmd, capture_output=True, text=True, cwd=cwd)
+        proc = subprocess.run(cmd, capture_output=True, text=True, cwd=work_dir)
         if proc.returncode != 0:
             raise RuntimeError(f"hipcc failed for {spec.show()}:\n{proc.stderr[-4000:]}")
-        if checked:
-            texts = [open(os.path.join(cwd, f)).read() for f in sorted(os.listdir(cwd))
-                     if f.endswith(".s") and "amdgcn" in f]
-            if not texts:
-                raise RuntimeError(f"no device assembly was kept for {spec.show()}")
-            check_generated_code(spec, texts[-1])
+        if work_dir:
+            stem = os.path.splitext(spec.template)[0]
+            kept = [f for f in os.listdir(work_dir)
+                    if f.endswith(".s") and "amdgcn" in f and f.startswith(stem + "-")]
+            if len(kept) != 1:
+                raise RuntimeError(f"expected one device assembly file for {spec.show()}, found {kept}")
+            asm_path = os.path.join(work_dir, kept[0])
+            if checked:
+                with open(asm_path) as f:
+                    check_generated_code(spec, f.read())
+            if dump_dir:
+                os.makedirs(dump_dir, exist_ok=True)
+                shutil.copyfile(asm_path, os.path.join(dump_dir, f"{stem}_{spec.key()}.s"))
     except Exception:
         if os.path.exists(tmp):
             os.remove(tmp)
         raise
     finally:
-        if scratch_dir:
-            shutil.rmtree(scratch_dir, ignore_errors=True)
+        if work_dir:
+            shutil.rmtree(work_dir, ignore_errors=True)
     os.replace(tmp, path)
     return path
 

@@ -15,10 +15,18 @@ import os
 DEFAULT_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "tuned_configs.json")
 
 
+INPUT_TAGS = {"normal": "", "uniform": "U(-1,1)"}
+
+
 def make_key(operator: str, shape, dtype: str = "float16", arch: str = "gfx950",
-             causal: bool = False) -> str:
+             causal: bool = False, inputs: str = "normal") -> str:
+    """`inputs`: the operand distribution the winner was measured on.  On a power-limited
+    board the fastest GEMM body depends on the operand statistics, so winners for U(-1,1)
+    operands are kept apart from those for the reference's N(0,1) (gemm_bench.py:26-31)."""
     dims = "x".join(str(int(d)) for d in shape)
-    return f"{operator}|{dims}|{dtype}{'|causal' if causal else ''}|{arch}"
+    tag = INPUT_TAGS[inputs]
+    return (f"{operator}|{dims}|{dtype}{'|causal' if causal else ''}"
+            f"{'|' + tag if tag else ''}|{arch}")
 
 
 def _config_class(operator: str):

@@ -43,6 +43,10 @@ def parse_args(argv=None):
                         help="with --cache: search again and replace the stored winner")
     parser.add_argument("--rounds", type=int, default=5,
                         help="interleaved timing rounds of the final comparison")
+    parser.add_argument("--timing", choices=["back_to_back", "events"], default="back_to_back",
+                        help="back_to_back: batches of launches between one event pair (what "
+                             "bench.py times); events: one event pair and one synchronisation "
+                             "per call, as the reference times")
     return parser.parse_args(argv)
 
 
@@ -66,7 +70,7 @@ def tune(args, shape, arch, arch_str, log):
     from deca_amd.Tuner import Tuner
 
     tuner = Tuner("flash_attn", arch, arch_str, args.top_n, args.jobs, args.finalists, args.rounds,
-                  cache_path=_cache_path(args), retune=args.retune)
+                  cache_path=_cache_path(args), retune=args.retune, timing=args.timing)
     return tuner.tune(*shape, log=log, causal=args.causal)
 
 

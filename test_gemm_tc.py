@@ -32,8 +32,10 @@ def parse_args(argv=None):
                         help="tune the square 2K-16K benchmark grid")
     parser.add_argument("--dtype", choices=["fp16", "bf16"], default="fp16",
                         help="type of A, B and C (accumulation is always fp32)")
-    parser.add_argument("--inputs", choices=["normal", "uniform"], default="normal",
-                        help="operand distribution: N(0,1) as the reference, or U(-1,1)")
+    parser.add_argument("--inputs", choices=["uniform", "normal"], default="uniform",
+                        help="operand distribution: U(-1,1), the benchmark's, or N(0,1) as the "
+                             "reference draws them (gemm_bench.py:26-31); winners are stored "
+                             "per distribution")
     parser.add_argument("--top_n", type=int, default=24,
                         help="number of ranked configs to compile and measure (0 = all)")
     parser.add_argument("--jobs", type=int, default=min(16, os.cpu_count() or 1),
@@ -47,6 +49,10 @@ def parse_args(argv=None):
                         help="with --cache: search again and replace the stored winner")
     parser.add_argument("--rounds", type=int, default=5,
                         help="interleaved timing rounds of the final comparison")
+    parser.add_argument("--timing", choices=["back_to_back", "events"], default="back_to_back",
+                        help="back_to_back: batches of launches between one event pair (what "
+                             "bench.py times); events: one event pair and one synchronisation "
+                             "per call, as the reference times")
     return parser.parse_args(argv)
 
 
@@ -62,7 +68,7 @@ def tune(args, shape, arch, arch_str, log):
     from deca_amd.Tuner import Tuner
 
     tuner = Tuner("GEMM", arch, arch_str, args.top_n, args.jobs, args.finalists, args.rounds,
-                  cache_path=_cache_path(args), retune=args.retune)
+                  cache_path=_cache_path(args), retune=args.retune, timing=args.timing)
     return tuner.tune(*shape, log=log, dtype=args.dtype, inputs=args.inputs)
 
 

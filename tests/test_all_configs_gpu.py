@@ -73,6 +73,40 @@ def _report(wrong):
         print(f"WRONG {name}: {err:.3e}", flush=True)
 
 
+MIN_LAUNCHED = 0.9
+
+
+def _load(spec, path, tally):
+    """The loaded kernel, or None for a config the tuner would drop as well: one whose
+    generated code the build step refused (`path is None`: only kernels that make promises
+    about their code can be), or whose code object the loader rejects (only kernels marked
+    `no_scratch`, when they spill).  Both are counted."""
+    from deca_amd.driver.driver import KernelRejected, load_kernel
+
+    meta = dict(spec.meta)
+    if path is None:
+        assert "accumulator_moves" in meta, f"an unchecked build was refused: {meta.get('cfg')}"
+        tally["refused"] += 1
+        return None
+    try:
+        kern = load_kernel(spec, path)
+    except KernelRejected as err:
+        assert meta.get("no_scratch"), f"rejected without the mark: {err}"
+        print(f"rejected {err}", flush=True)
+        tally["rejected"] += 1
+        return None
+    tally["launched"] += 1
+    return kern
+
+
+def _coverage(what, tally, total):
+    """What ran and what did not, on stdout; the sample must not shrink unnoticed."""
+    print(f"coverage {what}: {tally['launched']} launched, {tally['refused']} refused by the build "
+          f"step, {tally['rejected']} rejected by the loader, of {total}", flush=True)
+    assert sum(tally.values()) == total
+    assert tally["launched"] >= MIN_LAUNCHED * total, (what, tally)
+
+
 def _arch():
     from deca_amd.arch.MI355X import MI355X
 
@@ -82,7 +116,6 @@ def _arch():
 @pytest.mark.parametrize("B,H,S,D,causal", FA_SHAPES)
 def test_every_flash_attn_config(B, H, S, D, causal):
     from deca_amd import Solver
-    from deca_amd.driver.driver import load_kernel
     from deca_amd.kernels.attn_bench import make_qkv, math_attention
     from deca_amd.kernels.flash_attn_hip import make_flash_attn_fwd
 
@@ -93,20 +126,23 @@ def test_every_flash_attn_config(B, H, S, D, causal):
     paths = _build_all(specs)
     q, k, v = make_qkv(B, H, S, S, D)
     ref = math_attention(q, k, v, causal)
-    wrong = []
+    wrong, tally = [], {"launched": 0, "refused": 0, "rejected": 0}
     for cfg, spec, path in zip(configs, specs, paths):
+        kern = _load(spec, path, tally)
+        if kern is None:
+            continue
         o = torch.full_like(q, float("nan"))
-        _launch(f"fa B{B} H{H} S{S} D{D} causal={causal} {cfg}", load_kernel(spec, path), q, k, v, o)
+        _launch(f"fa B{B} H{H} S{S} D{D} causal={causal} {cfg}", kern, q, k, v, o)
         err = (o.float() - ref).abs().max().item()
         if not err <= 2e-3:
             wrong.append((str(cfg), err))
     _report(wrong)
+    _coverage(f"fa B{B} H{H} S{S} D{D} causal={causal}", tally, len(configs))
     assert not wrong, wrong[:8]
 
 
 @pytest.mark.parametrize("M,N,K", GEMM_SHAPES)
 def test_every_gemm_config(M, N, K):
-    from deca_amd.driver.driver import KernelRejected, load_kernel
     from deca_amd.kernels.gemm_bench import make_inputs
     from deca_amd.kernels.gemm_hip import make_gemm_tc
 
@@ -116,21 +152,18 @@ def test_every_gemm_config(M, N, K):
     a, b = make_inputs(M, N, K)
     ref = a.float() @ b.float()
     scale = ref.abs().max().item()
-    wrong = []
+    wrong, tally = [], {"launched": 0, "refused": 0, "rejected": 0}
     for cfg, spec, path in zip(configs, specs, paths):
-        if path is None:
+        kern = _load(spec, path, tally)
+        if kern is None:
             continue
         c = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
-        try:
-            kern = load_kernel(spec, path)
-        except KernelRejected as err:  # a build that spills: the tuner drops it the same way
-            print(f"rejected {err}", flush=True)
-            continue
         _launch(f"gemm {M}x{N}x{K} {cfg}", kern, a, b, c)
         err = (c.float() - ref).abs().max().item() / scale
         if not err <= 1e-2:
             wrong.append((str(cfg), err))
     _report(wrong)
+    _coverage(f"gemm {M}x{N}x{K}", tally, len(configs))
     assert not wrong, wrong[:8]
 
 

@@ -51,3 +51,45 @@ def test_build_refuses_a_kernel_whose_accumulators_the_compiler_moves(tmp_path):
     with pytest.raises(RuntimeError, match="accumulation-register moves"):
         build_kernel(_spec(2), None, str(tmp_path / "bad.hsaco"))
     assert not (tmp_path / "bad.hsaco").exists()
+
+
+def test_a_shared_dump_dir_cannot_lend_its_assembly_to_another_build(tmp_path):
+    """The checked assembly is this build's own: a dump directory that already holds other
+    kernels' files (one of them sorting after the GEMM's) changes neither the verdict nor
+    what is kept."""
+    from deca_amd.kernels.rowwise_hip import RowConfig, make_rowwise
+
+    dump = tmp_path / "dump"
+    dump.mkdir()
+    stale = dump / "rowwise-hip-amdgcn-amd-amdhsa-gfx950.s"
+    stale.write_text("\tv_accvgpr_mov_b32 a4, a8\n")           # would fail the check if it were read
+    (dump / "gemm-hip-amdgcn-amd-amdhsa-gfx950.s").write_text("stale\n")
+    spec = _spec(4)
+    build_kernel(spec, None, str(tmp_path / "g.hsaco"), str(dump))
+    kept = dump / f"gemm_{spec.key()}.s"
+    assert kept.exists() and "v_mfma_f32_16x16x32" in kept.read_text()
+    assert stale.read_text() == "\tv_accvgpr_mov_b32 a4, a8\n"
+    # a refused build leaves nothing of its own behind
+    bad = _spec(2)
+    with pytest.raises(RuntimeError, match="accumulation-register moves"):
+        build_kernel(bad, None, str(tmp_path / "b.hsaco"), str(dump))
+    assert not (dump / f"gemm_{bad.key()}.s").exists()
+    # unchecked builds keep their assembly the same way
+    row = make_rowwise("softmax", 256, 4096, "float16", RowConfig(128, 1, 8), 1e-6)
+    build_kernel(row, None, str(tmp_path / "r.hsaco"), str(dump))
+    assert (dump / f"rowwise_{row.key()}.s").exists()
+
+
+def test_checked_kernels_are_tied_to_the_validated_compiler(monkeypatch):
+    from deca_amd.kernels import build
+
+    spec = _spec(4)
+    assert build.hipcc_version().startswith(build.VALIDATED_HIPCC)
+    build.require_validated_hipcc(spec)
+    monkeypatch.setattr(build, "_hipcc_version", "HIP version: 9.9.0-deadbeef")
+    with pytest.raises(RuntimeError, match="validated with"):
+        build.require_validated_hipcc(spec)
+    with pytest.raises(RuntimeError, match="validated with"):
+        build.build_kernel(spec, None, "/nonexistent/never_written.hsaco".replace("/nonexistent", "/tmp"))
+    monkeypatch.setenv("DECA_ALLOW_UNCHECKED_HIPCC", "1")
+    build.require_validated_hipcc(spec)
