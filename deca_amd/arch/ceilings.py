@@ -262,7 +262,7 @@ def measure_sclk(out=sys.stdout):
     from deca_amd.kernels.gemm_hip import build_gemm_tc, make_gemm_tc
 
     n = 8192
-    cfg = tuned.lookup(tuned.make_key("GEMM", (n, n, n), "float16", "gfx950", False))
+    cfg = tuned.lookup(tuned.make_key("GEMM", (n, n, n), "float16", "gfx950", False, "uniform"))
     kern = build_gemm_tc(make_gemm_tc(n, n, n, cfg))
     print(f"idle: {_board_state()}", file=out, flush=True)
     makers = {"U(-1,1)": lambda: (2 * torch.rand(n, n, device="cuda") - 1).half(),

@@ -353,6 +353,17 @@ def fa_score(cfg, arch, shape, causal: bool = False) -> float:
         # the unrolled form of a tile this tight is expected to spill (3-67 registers measured)
         if register_fill(cfg, D) >= 0.95:
             pipe *= 0.965
+    # Measured on exhaustive runs of the S = 4096 shapes (config pairs that differ in nothing
+    # else): Q fragments re-read from LDS cost 1-5 % wherever the Q-in-registers twin fits its
+    # registers (they only win for tiles that would spill otherwise, which the solver's
+    # register limits already drop).  Requesting tiles two steps ahead instead of one pays for
+    # small K/V tiles, whose step is too short to cover a tile's latency (8 KiB: 0 ... +8 %,
+    # the D = 64 winner), is level to -3 % at 16 KiB and loses beyond.
+    if getattr(cfg, "q_in_smem", False):
+        pipe *= 0.975
+    if cfg.stages == 3:
+        tile_kib = cfg.Bc * D * 2 / 1024
+        pipe *= 1.015 if tile_kib <= 8 else (0.98 if tile_kib <= 16 else 0.95)
     if not getattr(cfg, "swizzle", True):
         pipe *= 0.5  # linear LDS rows: every fragment read is a multi-way bank conflict
     sync = 1.0 / (1.0 + getattr(arch, "fa_cta_sync_penalty", 0.0) * cfg.num_warps / 4 / wgs)

@@ -62,14 +62,18 @@ def attention_f32(q, k, v, scale=None, causal=False) -> np.ndarray:
     return out
 
 
-def flash_blockwise(q, k, v, scale=None, causal=False, Br=128, Bc=64, lazy_tau=0.0) -> np.ndarray:
+def flash_blockwise(q, k, v, scale=None, causal=False, Br=128, Bc=64, lazy_tau=0.0,
+                    max_every=1) -> np.ndarray:
     """The tiled online-softmax recurrence; returns fp32 values rounded to fp16.
 
     `lazy_tau` = 0 is the reference's update m' = max(m, rowmax S)
     (flash_attn_tir.py:419-428).  With `lazy_tau` > 0 the running max only
     follows a tile's max that lies more than 2^lazy_tau above it (in units of
     the exponent, (m' - m) * sl2): the HIP kernel's variant, which leaves O / l
-    the same quotient with p <= 2^lazy_tau."""
+    the same quotient with p <= 2^lazy_tau.  `max_every` > 1 looks at a tile's
+    max only in every `max_every`-th tile (a variant that was considered for the
+    kernel and is NOT safe: nothing bounds p in the tiles between, see
+    tests/test_oracle_attn.py)."""
     q = np.asarray(q, np.float32)
     k = np.asarray(k, np.float32)
     v = np.asarray(v, np.float32)
@@ -87,13 +91,15 @@ def flash_blockwise(q, k, v, scale=None, causal=False, Br=128, Bc=64, lazy_tau=0
                 l = np.zeros(qt.shape[0], np.float32)
                 o = np.zeros((qt.shape[0], D), np.float32)
                 kv_end = min(S_kv, -(-(q0 + Br) // Bc) * Bc) if causal else S_kv
-                for k0 in range(0, kv_end, Bc):
+                for tile, k0 in enumerate(range(0, kv_end, Bc)):
                     s = qt @ k[b, h, k0:k0 + Bc].T
                     if causal:
                         cols = np.arange(k0, k0 + s.shape[1])
                         s = np.where(cols[None, :] > rows[:, None], NEG_INF, s)
                     m_new = np.maximum(m, s.max(axis=-1))
-                    if lazy_tau > 0:
+                    if tile % max_every:
+                        m_new = m
+                    elif lazy_tau > 0:
                         m_new = np.where((m_new - m) * sl2 > np.float32(lazy_tau), m_new, m)
                     alpha = np.exp2((m - m_new) * sl2, dtype=np.float32)
                     p = np.exp2(s * sl2 - (m_new * sl2)[:, None], dtype=np.float32)

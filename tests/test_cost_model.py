@@ -141,3 +141,31 @@ def test_gemm_ranking_can_limit_the_tile_orders_per_tile_set():
     # the order of what is kept is still the score order
     scores = [cm.gemm_tc_score(c, ARCH, n, n, n) for c in spread]
     assert scores == sorted(scores, reverse=True)
+
+
+def test_rank_report_reads_the_drivers_output():
+    """The rank-quality table is made from the text the tuning drivers print."""
+    from deca_amd.cost_model import rank_report as rr
+
+    def rec(what, cfg, ms, thr, unit):
+        return f"{what} \n\t{cfg} \n\tcost time: {ms:.4f} ms, throughput: {thr:.2f} {unit}, max err: 1.00e-04\n"
+
+    text = "Detected GPU: X\nFind 244 FlashAttention configs, measuring 4\n"
+    fa = "FlashAttention(B=4, H=16, S_q=4096, S_kv=4096, D=128, float16)"
+    for cfg, thr in (("Br=256,Bc=128", 1000.0), ("Br=256,Bc=64", 1100.0), ("Br=128,Bc=64", 900.0),
+                     ("Br=64,Bc=64", 500.0)):
+        text += rec(fa, cfg, 0.5, thr, "TFLOPS")
+    text += "Br=32,Bc=32 is not a valid config: spills\n✅✅✅ 2026-01-01 [X]\n DeCA ...\n"
+    text += "Find 80 Softmax configs, measuring 2\n"
+    sm = "Softmax(M=16384, N=4096, float16)"
+    text += rec(sm, "tpr=256,rpb=2", 0.042, 6300.0, "GB/s") + rec(sm, "tpr=128,rpb=1", 0.05, 5300.0, "GB/s")
+    runs = rr.parse_runs(text)
+    assert [r["what"] for r in runs] == [fa, sm]
+    assert runs[0]["solutions"] == 244 and len(runs[0]["measured"]) == 4 and runs[1]["unit"] == "GB/s"
+    q = rr.quality(runs[0])
+    assert q["best_rank"] == 2 and q["best_cfg"] == "Br=256,Bc=64"
+    assert abs(q["first"] - 1000 / 1100) < 1e-9 and q["top3"] == 1.0
+    assert rr.spearman([4.0, 3.0, 2.0, 1.0]) == 1.0 and rr.spearman([1.0, 2.0, 3.0, 4.0]) == -1.0
+    assert rr.quality(runs[1])["best_rank"] == 1
+    lines = rr.table(runs).splitlines()
+    assert len(lines) == 4 and "| 244 | 4 | 2 |" in lines[2]

@@ -75,7 +75,13 @@ def test_flash_attn_closed_forms():
 
 
 def test_flash_attn_large_scores():
-    """Scores far from zero (|s| ~ 60) must not overflow the exponentials."""
+    """Scores far from zero (|s| ~ 60) must not overflow the exponentials.
+
+    With scores this peaked a row of P is close to one-hot and the output close to a single
+    row of V, |o| up to 4 and more, where the fp16 grid of the output alone is 3.9e-3 wide:
+    no fp16 result can meet an absolute 2e-3 there.  The gate is therefore 2e-3 relative to
+    max(1, |o|): the rounding of P to fp16 (2^-11 of each term) and of the output (2^-11 of
+    |o|) together stay below 1e-3 |o|, plus the 1e-4 the ordinary cases show."""
     from deca_amd.kernels.attn_bench import make_qkv_cpu
 
     B, H, Sq, Skv, D, _, cfg = FA_CASES[0]
@@ -84,7 +90,9 @@ def test_flash_attn_large_scores():
     k = (k.float() * 6).half()
     got = _f32(_run(B, H, Sq, Skv, D, False, cfg, q, k, v))
     assert np.isfinite(got).all()
-    assert np.abs(got - oa.attention_f32(_f32(q), _f32(k), _f32(v), None, False)).max() <= 4e-3
+    ref = oa.attention_f32(_f32(q), _f32(k), _f32(v), None, False)
+    assert np.abs(ref).max() > 3.0  # the regime the gate is written for
+    assert (np.abs(got - ref) <= GATE * np.maximum(1.0, np.abs(ref))).all()
 
 
 def _first_case(pipe, causal):

@@ -52,6 +52,28 @@ def test_blockwise_matches_plain_and_tiling_does_not_matter(causal):
     assert np.abs(one - many).max() < 2e-3
 
 
+def test_running_max_must_see_every_tile():
+    """Looking at the row max only in every second tile has no bound to stand on: the lazy
+    threshold bounds p by what the max of a tile *was seen* to be, and a tile that is not
+    looked at can lie any distance above it.  On keys that grow along the sequence the
+    skipped tiles push p past the fp16 range (65504) and the output is lost, while the
+    every-tile recurrence with the same threshold is within the gate."""
+    q, k, v = _qkv(1, 1, 64, 512, 64, seed=4)
+    k = k * np.linspace(0.2, 14.0, 512, dtype=np.float32)[None, None, :, None]
+    k = k.astype(np.float16).astype(np.float32)
+    ref = oa.attention_f32(q, k, v, None, False)
+    every = oa.flash_blockwise(q, k, v, None, False, Br=64, Bc=32, lazy_tau=8.0)
+    assert np.abs(every - ref).max() < 2e-3
+    with np.errstate(over="ignore", invalid="ignore"):
+        second = oa.flash_blockwise(q, k, v, None, False, Br=64, Bc=32, lazy_tau=8.0, max_every=2)
+    assert not np.isfinite(second).all() or np.abs(second - ref).max() > 2e-3
+    # the scores of a skipped tile do exceed the stale max by more than the fp16 exponent range
+    sl2 = 1.4426950408889634 / 8.0
+    s = np.einsum("bhqd,bhkd->bhqk", q, k)[0, 0] * sl2
+    seen = np.maximum.accumulate(s.reshape(64, 16, 32).max(-1), axis=1)
+    assert (s.reshape(64, 16, 32).max(-1)[:, 1:] - seen[:, :-1]).max() > 16 + 8
+
+
 @pytest.mark.parametrize("causal", [False, True])
 def test_lazy_running_max_is_the_same_quotient(causal):
     """The kernel's lazy running max against the reference's eager one: keys grow
