@@ -69,6 +69,33 @@ def workloads():
 
 DEFAULT_WORKLOAD = "rmsnorm_bf16_16384x4096"
 SPIN_UP_SECONDS = 0.3
+POWER_SECONDS = 0  # --power: seconds of board-state sampling per workload
+
+
+def _board(kern, sets):
+    """Shader clock and socket power (rocm-smi / amd-smi, one sample a second) while the
+    kernel repeats over `sets`; {} unless --power was given."""
+    if POWER_SECONDS <= 0:
+        return {}
+    import io
+    import re
+
+    from deca_amd.arch import ceilings
+
+    buf = io.StringIO()
+    ceilings._sample_while(lambda: [kern(*sets[i % len(sets)]) for i in range(50)], "board", buf,
+                           seconds=POWER_SECONDS + 1)
+    lines = buf.getvalue().splitlines()[1:]  # the first second still ramps
+    for line in lines:
+        print(f"[bench]   {line}", file=sys.stderr, flush=True)
+    mhz = [float(v) for line in lines for v in re.findall(r"\((\d+)Mhz\)", line)[:1]]
+    watts = [float(v) for line in lines for v in re.findall(r"SOCKET_POWER:\s*(\d+)", line)]
+    out = {}
+    if mhz:
+        out["sclk_mhz"] = [min(mhz), max(mhz)]
+    if watts:
+        out["socket_w"] = [min(watts), max(watts)]
+    return out
 
 
 def _spec(wl):
@@ -146,6 +173,7 @@ def run_rowwise(wl, steps, warmup, with_cpu):
             "algorithmic_bytes": nbytes, "buffer_sets": nsets,
         },
     }
+    res["roofline"].update(_board(kern, sets))
     if with_cpu:
         res["cpu_baseline"] = cpu_baseline(wl)
     del sets
@@ -194,6 +222,7 @@ def run_gemm(wl, steps, warmup, with_cpu):
     c = torch.empty(M, N, dtype=tdt, device="cuda")
     wall, t_k = _timed_steps(kern, [(a, b, c)], steps, warmup)
     flops = gemm_flops(M, N, K)
+    board = _board(kern, [(a, b, c)])
     # the same kernel on the reference's operand distribution, N(0,1) (gemm_bench.py:26-31):
     # the board is power-limited and the rate follows the operand statistics
     a, b = make_inputs(M, N, K, seed=0, dist="normal", dtype=tdt)
@@ -209,6 +238,7 @@ def run_gemm(wl, steps, warmup, with_cpu):
                      "traffic": None, "kernel_us": t_k * 1e6, "algorithmic_flops": flops,
                      "achieved_normal_inputs": flops / t_n01 / 1e12},
     }
+    res["roofline"].update(board)
     if with_cpu:
         res["cpu_baseline"] = cpu_baseline(wl)
     del a, b, c
@@ -237,6 +267,7 @@ def run_fa(wl, steps, warmup, with_cpu):
                      "unit": "TFLOP/s", "frac": flops / t_k / 1e12 / MFMA_PEAK_TFLOPS,
                      "traffic": None, "kernel_us": t_k * 1e6, "algorithmic_flops": flops},
     }
+    res["roofline"].update(_board(kern, [(q, k, v, o)]))
     if with_cpu:
         res["cpu_baseline"] = cpu_baseline(wl)
     del q, k, v, o
@@ -284,6 +315,9 @@ def _compact(res):
     }
     if "achieved_normal_inputs" in rf:
         row["achieved_n01"] = round(rf["achieved_normal_inputs"], 1)
+    for key in ("sclk_mhz", "socket_w"):
+        if key in rf:
+            row[key] = rf[key]
     target = TARGET_FRAC.get(res["workload"])
     if target is not None:
         row["target_frac"] = target
@@ -371,6 +405,9 @@ def main():
                          "--workload instead of its stored winner; implies --no-extra")
     ap.add_argument("--no-extra", action="store_true", help="only the headline workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--power", type=int, default=0, metavar="SECONDS",
+                    help="after timing a workload, sample shader clock and socket power once a "
+                         "second for this long while its kernel repeats (roofline.sclk_mhz / socket_w)")
     ap.add_argument("--full-out", default=os.path.join(ROOT, "gpurun_out", "bench_full.json"),
                     metavar="PATH", help="file for the full per-workload records ('' for none)")
     args = ap.parse_args()
@@ -383,6 +420,8 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs a GPU (the kernels have no host path)", file=sys.stderr)
         sys.exit(1)
+    global POWER_SECONDS
+    POWER_SECONDS = args.power
     wls = workloads()
     if args.kernel_config:
         from deca_amd import tuned

@@ -11,6 +11,8 @@ with traces):
     fetch   --pmc FETCH_SIZE                             20 steps
     write   --pmc WRITE_SIZE                             20 steps
     sq      --pmc SQ_* GRBM_GUI_ACTIVE (matrix kernels)  20 steps
+    board   no profiler: bench.py --power 4 (shader clock and socket power, sampled once a
+            second while the kernel repeats)
 
 each over `python3 bench.py --workload WORKLOAD --no-extra --no-cpu`.
 `summarise` turns their CSV files into `profiles/<kernel>_<workload>.md` and
@@ -54,9 +56,12 @@ def kernel_of(workload: str) -> str:
     return KERNEL_OF[workload.split("_")[0]]
 
 
-def passes(workload: str) -> dict:
-    """name -> (rocprofv3 options, bench.py options) of the profiler passes."""
+def passes(workload: str, kernel_config: str | None = None) -> dict:
+    """name -> (rocprofv3 options, bench.py options) of the profiler passes; with
+    `kernel_config`, over that configuration instead of the stored winner."""
     bench = ["--workload", workload, "--no-extra", "--no-cpu", "--full-out", ""]
+    if kernel_config:
+        bench += ["--kernel-config", kernel_config]
     short = bench + ["--steps", "20", "--warmup", "2"]
     out = {
         "trace": (["--kernel-trace", "--stats"], bench + ["--steps", "100", "--warmup", "10"]),
@@ -65,21 +70,24 @@ def passes(workload: str) -> dict:
     }
     if kernel_of(workload) != "rowwise":
         out["sq"] = (["--pmc", *SQ_COUNTERS], short)
+    out["board"] = (None, short + ["--power", "4"])
     return out
 
 
-def command(workload: str, name: str, out_dir: str) -> list:
-    prof, bench = passes(workload)[name]
+def command(workload: str, name: str, out_dir: str, kernel_config: str | None = None) -> list:
+    prof, bench = passes(workload, kernel_config)[name]
+    if prof is None:
+        return ["python3", os.path.join(ROOT, "bench.py"), *bench]
     return ["rocprofv3", *prof, "-d", os.path.join(out_dir, name), "-o", "out", "--output-format", "csv",
             "--", "python3", os.path.join(ROOT, "bench.py"), *bench]
 
 
-def run(workload: str, out_dir: str, timeout_s: int = 200) -> None:
+def run(workload: str, out_dir: str, timeout_s: int = 200, kernel_config: str | None = None) -> None:
     """Runs the passes one after the other; stops at the first that fails."""
     os.makedirs(out_dir, exist_ok=True)
     env = dict(os.environ, TMPDIR="/tmp")
-    for name in passes(workload):
-        cmd = command(workload, name, out_dir)
+    for name in passes(workload, kernel_config):
+        cmd = command(workload, name, out_dir, kernel_config)
         print("[profile]", " ".join(cmd), flush=True)
         with open(os.path.join(out_dir, f"{name}.log"), "w") as log:
             done = subprocess.run(cmd, cwd="/tmp", env=env, stdout=log, stderr=subprocess.STDOUT,
@@ -173,7 +181,7 @@ def matrix_pipe(sq_rows: list) -> dict:
 # ---------------------------------------------------------------------------
 # the summary
 # ---------------------------------------------------------------------------
-def summary_text(workload: str, out_dir: str) -> tuple:
+def summary_text(workload: str, out_dir: str, kernel_config: str | None = None) -> tuple:
     """(markdown text, entry for measured_traffic.json) from the passes' output."""
     kern = kernel_of(workload)
     rowwise = kern == "rowwise"
@@ -186,12 +194,16 @@ def summary_text(workload: str, out_dir: str) -> tuple:
     write = counter_means(_rows(os.path.join(out_dir, "write", "out_counter_collection.csv")))
 
     def rel(cmd):
-        return " ".join(cmd).replace(ROOT + os.sep, "").replace(out_dir, "<out>")
+        words = [f"'{w}'" if "," in w else w for w in cmd]
+        return " ".join(words).replace(ROOT + os.sep, "").replace(out_dir, "<out>")
 
-    t = [f"# rocprofv3 summary: `{kern}.hip` on workload `{workload}`", "",
-         f"Made by `python -m deca_amd.arch.profile run {workload}` and `... summarise {workload}` "
-         "on a 1-GPU MI355X box; the passes it runs (from `/tmp`, `TMPDIR=/tmp`):", "", "```"]
-    t += [rel(command(workload, name, out_dir)) for name in passes(workload)]
+    extra = f" --kernel-config '{kernel_config}'" if kernel_config else ""
+    t = [f"# rocprofv3 summary: `{kern}.hip` on workload `{workload}`"
+         + (f", configuration `{kernel_config}`" if kernel_config else ""), "",
+         f"Made by `python -m deca_amd.arch.profile run {workload}{extra}` and `... summarise "
+         f"{workload}{extra}` on a 1-GPU MI355X box; the passes it runs (from `/tmp`, `TMPDIR=/tmp`):",
+         "", "```"]
+    t += [rel(command(workload, name, out_dir, kernel_config)) for name in passes(workload, kernel_config)]
     t += ["```", "", "## Kernel trace statistics (top kernels)", "",
           "| kernel | calls | avg ns | min ns | max ns | % of GPU time |", "|---|---|---|---|---|---|"]
     for r in stats[:4]:
@@ -247,6 +259,16 @@ def summary_text(workload: str, out_dir: str) -> tuple:
               f"| SQ_INSTS_VALU (includes MFMA) per MFMA | {mp['valu_per_mfma']:.2f} |",
               f"| SQ_INSTS_LDS per MFMA | {mp['lds_per_mfma']:.2f} |",
               f"| SQ_LDS_BANK_CONFLICT cycles | {mp['bank_conflict_cycles']:.4g} |"]
+    board_log = os.path.join(out_dir, "board.log")
+    board = bench_record(board_log) if os.path.exists(board_log) else None
+    if board and "socket_w" in board["roofline"]:
+        rf = board["roofline"]
+        clk = rf.get("sclk_mhz", [0, 0])
+        t += ["", "## Board state while the kernel repeats (the `board` pass: rocm-smi / amd-smi, one "
+              "sample a second for 4 s)", "",
+              f"Shader clock {clk[0]:.0f}-{clk[1]:.0f} MHz, socket power {rf['socket_w'][0]:.0f}-"
+              f"{rf['socket_w'][1]:.0f} W; the launches timed just before ran at {rf['achieved']:.0f} "
+              f"{rf['unit']}."]
     entry = {"config": rec["config"]["kernel_config"], "fetch_size_kib": round(mine_f, 1),
              "write_size_kib": round(mine_w, 1), "fetch_scale": FETCH_SCALE, "write_scale": WRITE_SCALE,
              "traffic_bytes": total}
@@ -254,12 +276,18 @@ def summary_text(workload: str, out_dir: str) -> tuple:
 
 
 def summarise(workload: str, out_dir: str, profiles_dir: str | None = None,
-              traffic_path: str | None = None) -> str:
-    text, entry = summary_text(workload, out_dir)
+              traffic_path: str | None = None, kernel_config: str | None = None,
+              tag: str | None = None) -> str:
+    """Writes the summary; the traffic table only takes figures of the stored winners (a
+    run over another `kernel_config` is written as `..._<tag>.md` and recorded nowhere)."""
+    text, entry = summary_text(workload, out_dir, kernel_config)
     profiles_dir = profiles_dir or os.path.join(ROOT, "profiles")
-    path = os.path.join(profiles_dir, f"{kernel_of(workload)}_{workload}.md")
+    name = f"{kernel_of(workload)}_{workload}" + (f"_{tag}" if kernel_config else "")
+    path = os.path.join(profiles_dir, name + ".md")
     with open(path, "w") as f:
         f.write(text)
+    if kernel_config:
+        return path
     traffic_path = traffic_path or os.path.join(PKG, "measured_traffic.json")
     table = {"workloads": {}}
     if os.path.exists(traffic_path):
@@ -277,13 +305,17 @@ def main(argv=None):
     ap.add_argument("action", choices=["run", "summarise"])
     ap.add_argument("workload")
     ap.add_argument("--out", default=None, help="directory of the passes' output "
-                                                "(default gpurun_out/prof_<workload>)")
+                                                "(default gpurun_out/prof_<workload>[_<tag>])")
+    ap.add_argument("--kernel-config", default=None, metavar="TEXT",
+                    help="profile this configuration instead of the stored winner")
+    ap.add_argument("--tag", default="variant", help="with --kernel-config: suffix of the summary's name")
     args = ap.parse_args(argv)
-    out_dir = os.path.abspath(args.out or os.path.join(ROOT, "gpurun_out", f"prof_{args.workload}"))
+    default = f"prof_{args.workload}" + (f"_{args.tag}" if args.kernel_config else "")
+    out_dir = os.path.abspath(args.out or os.path.join(ROOT, "gpurun_out", default))
     if args.action == "run":
-        run(args.workload, out_dir)
+        run(args.workload, out_dir, kernel_config=args.kernel_config)
     else:
-        print("wrote", summarise(args.workload, out_dir))
+        print("wrote", summarise(args.workload, out_dir, kernel_config=args.kernel_config, tag=args.tag))
 
 
 if __name__ == "__main__":

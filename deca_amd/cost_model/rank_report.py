@@ -1,6 +1,7 @@
 """Rank quality of the cost models, from the tuning drivers' own output.
 
     python -m deca_amd.cost_model.rank_report LOG [LOG ...] > profiles/rank_quality.md
+    python -m deca_amd.cost_model.rank_report --pairs q_smem=0:q_smem=1 stages=2:stages=3 -- LOG ...
 
 A driver (`test_gemm_tc.py`, `test_rowwise.py`, `test_flash_attn.py`) prints one
 record per measured configuration, in the order the cost model ranked them, and
@@ -75,15 +76,56 @@ def table(runs: list) -> str:
     return "\n".join(rows)
 
 
+def pair_effects(run: dict, old: str, new: str) -> dict:
+    """What one field of the configuration does, everything else equal: over all measured
+    pairs of configurations whose text differs only in `old` -> `new` (e.g. "stages=2",
+    "stages=3"), the ratios new / old, the pair with the fastest `new` member, and the
+    same ratios among pairs whose better member is within 10 % of the run's best."""
+    thr = dict(run["measured"])
+    best = max(thr.values())
+    pairs = [(c, c.replace(old, new)) for c in thr if old in c.split(",") and c.replace(old, new) in thr]
+    ratios = sorted(thr[b] / thr[a] for a, b in pairs)
+    near = sorted(thr[b] / thr[a] for a, b in pairs if max(thr[a], thr[b]) >= 0.9 * best)
+    top = max(pairs, key=lambda ab: thr[ab[1]], default=None)
+
+    def mid(v):
+        return v[len(v) // 2] if v else float("nan")
+
+    return {"pairs": len(pairs), "median": mid(ratios), "min": ratios[0] if ratios else float("nan"),
+            "max": ratios[-1] if ratios else float("nan"), "near_pairs": len(near), "near_median": mid(near),
+            "near_min": near[0] if near else float("nan"), "near_max": near[-1] if near else float("nan"),
+            "top": None if top is None else (top[1], thr[top[1]], thr[top[0]]), "best": best}
+
+
+def pairs_table(runs: list, fields: list) -> str:
+    rows = ["| tuned shape | field | pairs | new / old: median (min ... max) | ... among pairs within "
+            "10 % of the best | fastest config with the new value | its twin with the old | "
+            "best of the run |", "|---|---|---|---|---|---|---|---|"]
+    for run in runs:
+        for field in fields:
+            old, new = field.split(":")
+            e = pair_effects(run, old, new)
+            top = "-" if e["top"] is None else f"`{e['top'][0]}` {e['top'][1]:.1f}"
+            twin = "-" if e["top"] is None else f"{e['top'][2]:.1f}"
+            rows.append(f"| {run['what']} | {old} -> {new} | {e['pairs']} | {e['median']:.3f} "
+                        f"({e['min']:.3f} ... {e['max']:.3f}) | {e['near_pairs']} pairs: {e['near_median']:.3f} "
+                        f"({e['near_min']:.3f} ... {e['near_max']:.3f}) | {top} | {twin} | {e['best']:.1f} |")
+    return "\n".join(rows)
+
+
 def main(argv=None):
-    paths = (argv if argv is not None else sys.argv[1:])
-    if not paths:
+    args = list(argv if argv is not None else sys.argv[1:])
+    fields = []
+    if args and args[0] == "--pairs":
+        cut = args.index("--")
+        fields, args = args[1:cut], args[cut + 1:]
+    if not args:
         raise SystemExit(__doc__)
     runs = []
-    for p in paths:
+    for p in args:
         with open(p) as f:
             runs += parse_runs(f.read())
-    print(table(runs))
+    print(pairs_table(runs, fields) if fields else table(runs))
 
 
 if __name__ == "__main__":

@@ -57,7 +57,11 @@ def test_passes_keep_counters_apart_from_traces():
     for wl in ("gemm_fp16_8192", "softmax_fp16_16384x4096", "fa_fp16_b4h16s4096d128_causal"):
         p = profile.passes(wl)
         assert ("sq" in p) == (profile.kernel_of(wl) != "rowwise")
+        assert p["board"][0] is None and p["board"][1][-2:] == ["--power", "4"]
+        assert profile.command(wl, "board", "/x")[0] == "python3"
         for name, (prof, bench) in p.items():
+            if prof is None:
+                continue
             assert ("--pmc" in prof) != ("--kernel-trace" in prof)
             assert bench[:2] == ["--workload", wl] and "--no-cpu" in bench
             cmd = profile.command(wl, name, "/x")
@@ -97,7 +101,16 @@ def test_summary_and_traffic_table(tmp_path):
     text = open(profile.summarise("gemm_fp16_2048", out, str(prof_dir), traffic)).read()
     assert "not derived" in text and "GHz (2.4 GHz nominal)" not in text
     out = _passes(tmp_path, "fa_fp16_b4h16s4096d128", 480_000)
+    with open(os.path.join(out, "board.log"), "w") as f:
+        f.write(json.dumps({"roofline": {"sclk_mhz": [2100.0, 2140.0], "socket_w": [1330.0, 1350.0],
+                                         "achieved": 1140.2, "unit": "TFLOP/s"}}) + "\n")
     text = open(profile.summarise("fa_fp16_b4h16s4096d128", out, str(prof_dir), traffic)).read()
     assert "2.00 GHz" in text and "16x16x32" in text
+    assert "Shader clock 2100-2140 MHz, socket power 1330-1350 W" in text
+    # another configuration than the stored winner: its own file, nothing recorded
+    path = profile.summarise("fa_fp16_b4h16s4096d128", out, str(prof_dir), traffic,
+                             kernel_config="Br=256,Bc=64,q_smem=1", tag="q_smem")
+    assert path.endswith("flash_attn_fa_fp16_b4h16s4096d128_q_smem.md")
+    assert "--kernel-config 'Br=256,Bc=64,q_smem=1'" in open(path).read()
     assert set(json.load(open(traffic))["workloads"]) == {
         "softmax_fp16_16384x4096", "gemm_fp16_2048", "fa_fp16_b4h16s4096d128"}

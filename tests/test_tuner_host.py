@@ -208,6 +208,72 @@ def test_tuned_table_roundtrip(tmp_path):
     assert len(bench.workloads()) == 13
 
 
+def test_shipped_winners_come_from_the_tuner():
+    """Every entry of the shipped table was written by `Tuner.tune` (the drivers'
+    `--cache --retune`), timed back to back, after measuring a real share of the solver's
+    list; the GEMM entries bench.py uses are the ones tuned on its U(-1,1) operands."""
+    import bench
+    from deca_amd import tuned
+
+    table = tuned.load()
+    for key, entry in table.items():
+        assert entry.get("method") == "tuner", key
+        assert entry.get("timing") == "back_to_back", key
+        assert 1 <= entry["rank"] <= entry["candidates"] <= entry["solutions"], key
+        assert entry["candidates"] >= min(16, entry["solutions"]), key
+        assert entry["torch_throughput"] > 0 and entry["runtime_ms"] > 0, key
+        if key.startswith("GEMM"):
+            assert ("|U(-1,1)|" in key) == (entry.get("inputs") == "U(-1,1)"), key
+    # bench.py finds all of its 13 workloads there (it raises on a missing key)
+    assert len(bench.workloads()) == 13
+    bf16 = table[tuned.make_key("GEMM", (8192, 8192, 8192), "bfloat16", "gfx950", False, "uniform")]
+    # the bf16 winner was searched with the 16x16x32 and accumulation-register bodies on offer
+    assert bf16["candidates"] >= 24
+
+
+def test_tuner_timing_modes(monkeypatch):
+    """`timing` reaches RuntimeMod, and the two procedures differ as documented: one event
+    pair per call, or batches between one pair."""
+    import pytest as _pytest
+
+    from deca_amd.kernels import attn_bench as ab
+    from deca_amd.operators import Softmax
+    from deca_amd.RuntimeMod import RuntimeMod
+    from deca_amd.Tuner import Tuner
+
+    assert ab.TIMINGS == ("events", "back_to_back")
+    assert Tuner("softmax", arch=object(), arch_str="gfx950").timing == "back_to_back"
+    assert Tuner("softmax", arch=object(), arch_str="gfx950", timing="events").timing == "events"
+    with _pytest.raises(AssertionError):
+        Tuner("softmax", arch=object(), arch_str="gfx950", timing="wall")
+    rt = RuntimeMod(Softmax(64, 128, "float16"), None, True, RowConfig(16, 4, 8), timing="back_to_back")
+    assert rt.timing == "back_to_back" and RuntimeMod(rt.operator, None, True, None).timing == "events"
+    # bench_back_to_back: warm-up by time, then `batches` batches sized from the settled time
+    calls = []
+
+    def timed(n):
+        calls.append(n)
+        return 1e-3
+
+    monkeypatch.setattr(ab.time, "perf_counter", iter([0.0, 0.1, 0.2, 0.4, 0.5]).__next__)
+    t = ab.bench_back_to_back(timed, warmup_s=0.3, measure_s=0.3, min_iters=20, batches=3)
+    assert t == 1e-3 and calls[0] == 4 and calls[-3:] == [100, 100, 100]
+    seen = ab.bench_interleaved_batches.__doc__
+    assert "batch timers" in seen
+
+
+def test_winners_are_kept_per_operand_distribution(tmp_path):
+    from deca_amd import tuned
+    from deca_amd.kernels.gemm_hip import GemmConfig
+
+    n01 = tuned.make_key("GEMM", (4096, 4096, 4096), "float16")
+    uni = tuned.make_key("GEMM", (4096, 4096, 4096), "float16", "gfx950", False, "uniform")
+    assert n01 == "GEMM|4096x4096x4096|float16|gfx950" and uni == "GEMM|4096x4096x4096|float16|U(-1,1)|gfx950"
+    path = str(tmp_path / "t.json")
+    tuned.store(uni, GemmConfig(256, 256, 64, 128, 64, 2, 0), 1300.0, "TFLOPS", path, inputs="U(-1,1)")
+    assert tuned.lookup(n01, path) is None and tuned.lookup(uni, path) is not None
+
+
 def test_shipped_winners_are_solver_candidates():
     """Every entry of the shipped table is a configuration its solver still emits for
     that shape (a rule added to a solver must not leave a stale winner behind)."""
