@@ -351,7 +351,7 @@ def solve_gemm_tc(arch, M: int, N: int, K: int, type_size: int = 2, count: int =
     """
     from dataclasses import replace
 
-    from deca_amd.kernels.gemm_hip import GemmConfig, agpr_split_fits, check_config
+    from deca_amd.kernels.gemm_hip import GemmConfig, agpr_split_fits, check_config, default_spread
 
     tiles = _enumerate(GEMM_DOMAINS, _gemm_constraints(arch, M, N, K, type_size), count, backend)
     results = []
@@ -376,6 +376,9 @@ def solve_gemm_tc(arch, M: int, N: int, K: int, type_size: int = 2, count: int =
                 # the accumulators in accumulation registers, where both halves of the
                 # register file have room for their share
                 cands += [replace(c, agpr=True) for c in cands if agpr_split_fits(c)]
+                # the tile loads dealt over the MFMA groups instead of issued in a burst
+                if default_spread(cfg):
+                    cands += [replace(c, spread=default_spread(cfg)) for c in cands]
             for cand in cands:
                 if ras == 0 or cand.tail:
                     try:

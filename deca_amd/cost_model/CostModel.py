@@ -244,6 +244,13 @@ def gemm_tc_score(cfg, arch, M: int, N: int, K: int) -> float:
         # at 4096^3 and 8192^3)
         if getattr(cfg, "agpr", False):
             form += 0.03
+        # tile loads dealt over the MFMA groups: the more loads a wave issues per K-tile, the
+        # longer the queue at the load path that the burst form makes every wave stand in
+        # (measured with 8 loads per lane and K-tile: +2 % at 4096^3, +6 % at 8192^3, +7.5 %
+        # at 16384^3; with 4: +1 %)
+        if getattr(cfg, "spread", 0):
+            loads = (cfg.BM * cfg.BK + cfg.BK * cfg.BN) // 8 // cfg.threads
+            form += 0.005 * loads
 
     return form * wave_eff * hiding * pipe * sync_eff * staged / ((t_flop + t_epi) / t_mma)
 
@@ -261,7 +268,7 @@ def rank_gemm_configs(configs, arch, M: int, N: int, K: int, top_n: int | None =
 
         seen, kept = {}, []
         for c in ranked:
-            key = replace(c, raster=1, early=0, agpr=False)
+            key = replace(c, raster=1, early=0, agpr=False, spread=0)
             seen[key] = seen.get(key, 0) + 1
             if seen[key] <= per_tile:
                 kept.append(c)

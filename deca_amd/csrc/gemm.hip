@@ -65,6 +65,12 @@
 #ifndef DECA_ACC_AGPR
 #define DECA_ACC_AGPR 0  // 16x16x32 body: 1 keeps the accumulators in accumulation registers (MFMAs as inline asm)
 #endif
+#ifndef DECA_DMA_SPREAD
+#define DECA_DMA_SPREAD 0  // 16x16x32 body: MFMA groups of a K-tile over which its global->LDS loads are dealt (0: one burst)
+#endif
+#ifndef DECA_DMA_FIRST
+#define DECA_DMA_FIRST 0  // ... and the number of groups behind the barrier that pass before the first load
+#endif
 #ifndef DECA_EARLY_GROUPS
 #define DECA_EARLY_GROUPS 0  // 16x16x32 body: MFMA groups of a K-tile's last k-step issued before its barrier
 #endif

@@ -68,6 +68,13 @@ class GemmConfig:
     # as inline assembly (about 3 % faster than the builtin form; the build step checks the
     # generated code, see `accumulator_moves`)
     agpr: bool = False
+    # 16x16x32 body: the global->LDS loads of a tile are dealt over this many MFMA groups
+    # instead of issued in one burst at the top of a K-tile (0).  All waves of a workgroup
+    # leave the K-tile barrier together and queue up at the CU's one load path (a 64-lane x
+    # 16-byte load per 16 clocks); a wave in that queue issues no MFMA.  The window of a
+    # tile opens one group behind the barrier that frees its ring slot and runs into the
+    # next K-tile (measured: +2 % at 4096^3, +6 % at 8192^3, +7.5 % at 16384^3 with 6).
+    spread: int = 0
 
     @property
     def num_warps(self) -> int:
@@ -90,7 +97,24 @@ class GemmConfig:
             + (f",mfma={self.mfma}" if self.mfma != 32 else "")
             + (f",early={self.early}" if self.early else "")
             + (",agpr=1" if self.agpr else "")
+            + (f",spread={self.spread}" if self.spread else "")
         )
+
+
+# Groups behind a K-tile's barrier that pass before the first load of the spread window.
+SPREAD_FIRST = 1
+
+
+def mfma_groups_per_ktile(cfg: GemmConfig) -> int:
+    """MFMA groups (one row block against every column block) of a K-tile in the 16x16x32 body."""
+    return (cfg.BK // 32) * (cfg.warp_m // 16)
+
+
+def default_spread(cfg: GemmConfig) -> int:
+    """The window the solver offers for a tile: 6 groups where a K-tile has 12 or more
+    (measured best of 2..12 for 256 x 256 x 64 tiles), 3 where it has 6 or more, else none."""
+    groups = mfma_groups_per_ktile(cfg)
+    return 6 if groups >= 12 else (3 if groups >= 6 else 0)
 
 
 def pipeline_smem_bytes(cfg: GemmConfig) -> int:
@@ -195,8 +219,9 @@ def check_config(cfg: GemmConfig, M: int, N: int, K: int, max_smem: int = MAX_LD
         # 64 accumulator tiles of 16 x 16 per wave: hipcc fills all 256 accumulation and
         # all 256 vector registers and still spills 30-170 inside the loop (8x slower)
         assert (cfg.warp_m // 16) * (cfg.warp_n // 16) <= 32
+        assert 0 <= cfg.spread <= mfma_groups_per_ktile(cfg) - SPREAD_FIRST
     else:
-        assert cfg.early == 0 and not cfg.agpr
+        assert cfg.early == 0 and not cfg.agpr and cfg.spread == 0
     assert cfg.warp_m % MFMA_M == 0 and cfg.warp_n % MFMA_M == 0
     assert cfg.BM % cfg.warp_m == 0 and cfg.BN % cfg.warp_n == 0
     assert cfg.BN >= 64
@@ -259,6 +284,9 @@ def make_gemm_tc(M: int, N: int, K: int, cfg: GemmConfig, dtype: str = "float16"
         defines["DECA_EARLY_GROUPS"] = cfg.early
     if cfg.agpr:
         defines["DECA_ACC_AGPR"] = 1
+    if cfg.spread:
+        defines["DECA_DMA_SPREAD"] = cfg.spread
+        defines["DECA_DMA_FIRST"] = SPREAD_FIRST
     workgroups = (M // cfg.BM) * (N // cfg.BN)
     if cfg.tail:
         r = tail_tiles(cfg, M, N)
@@ -269,9 +297,10 @@ def make_gemm_tc(M: int, N: int, K: int, cfg: GemmConfig, dtype: str = "float16"
         TEMPLATE, defines, grid=(workgroups, 1, 1), block=(cfg.threads, 1, 1),
         nargs=3, options=FAST_MATH_OPTIONS,
         # the direct-load ring waits with vmcnt(n > 0) once it is deeper than two tiles
-        # (the quarter tiles of `tail` always are): the loader refuses a build that spills
+        # (the quarter tiles of `tail` always are; with `spread` the prologue does, for the
+        # head of the second tile): the loader refuses a build that spills
         meta={"cfg": str(cfg), "dtype": dtype,
-              "no_scratch": bool(cfg.direct and (cfg.stages > 2 or cfg.tail)),
+              "no_scratch": bool(cfg.direct and (cfg.stages > 2 or cfg.tail or cfg.spread)),
               **({"accumulator_moves": accumulator_moves(cfg)} if cfg.agpr else {})},
     )
 

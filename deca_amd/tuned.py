@@ -90,7 +90,8 @@ def parse_config(operator: str, text: str):
                       raster=int(pairs.pop("raster")), epi_smem=bool(int(pairs.pop("epi_smem"))),
                       xcd=bool(int(pairs.pop("xcd", 1))), direct=bool(int(pairs.pop("direct", 1))),
                       tail=bool(int(pairs.pop("tail", 0))), mfma=int(pairs.pop("mfma", 32)),
-                      early=int(pairs.pop("early", 0)), agpr=bool(int(pairs.pop("agpr", 0))))
+                      early=int(pairs.pop("early", 0)), agpr=bool(int(pairs.pop("agpr", 0))),
+                      spread=int(pairs.pop("spread", 0)))
     elif operator in ("softmax", "rmsnorm"):
         fields.update(threads_per_row=int(pairs.pop("tpr")), rows_per_block=int(pairs.pop("rpb")),
                       vec=int(pairs.pop("vec")), mode=pairs.pop("mode"),

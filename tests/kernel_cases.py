@@ -107,6 +107,20 @@ GEMM_CASES = [
     (384, 640, 1088, GemmConfig(128, 128, 64, 64, 32, 5, 1, True, False, True, mfma=16, early=2, agpr=True)),
     (256, 256, 128, GemmConfig(64, 64, 64, 32, 32, 2, 1, False, False, True, mfma=16, agpr=True)),
     (3072, 3072, 256, GemmConfig(128, 128, 64, 64, 64, 2, 0, True, True, True, True, mfma=16, agpr=True)),
+    # ... with the tile loads dealt over the MFMA groups (`spread`): windows shorter and longer
+    # than the groups behind the barrier, rings of 2..5, one k-step per K-tile (two tiles per
+    # loop iteration), builtin and accumulation-register MFMAs, the block order and the tail
+    (512, 512, 512, GemmConfig(256, 256, 64, 128, 64, 2, 1, True, False, True, mfma=16, early=4, agpr=True, spread=6)),
+    (512, 512, 512, GemmConfig(256, 256, 64, 128, 64, 2, 2, False, False, True, mfma=16, spread=2)),
+    (512, 512, 512, GemmConfig(256, 256, 64, 128, 64, 2, 1, True, False, True, mfma=16, early=6, spread=15)),
+    (512, 1024, 256, GemmConfig(256, 256, 32, 128, 64, 3, 2, True, True, True, mfma=16, early=4, spread=6)),
+    (512, 512, 512, GemmConfig(256, 256, 32, 64, 128, 5, 1, True, False, True, mfma=16, early=3, spread=3)),
+    (384, 640, 1088, GemmConfig(128, 128, 64, 64, 32, 4, 1, True, False, True, mfma=16, early=2, agpr=True, spread=3)),
+    (256, 256, 128, GemmConfig(64, 64, 64, 32, 32, 2, 1, False, False, True, mfma=16, spread=3)),
+    (128, 192, 64, GemmConfig(64, 64, 32, 32, 64, 2, 2, False, False, True, mfma=16, spread=1)),
+    (3072, 4096, 128, GemmConfig(128, 128, 64, 64, 64, 2, 0, False, True, True, mfma=16, early=2, spread=3)),
+    (3072, 3072, 256, GemmConfig(128, 128, 64, 64, 64, 2, 0, True, True, True, True, mfma=16, agpr=True, spread=6)),
+    (3072, 3072, 256, GemmConfig(128, 128, 64, 64, 64, 2, 4, True, True, True, True, mfma=16, early=2, spread=3)),
     # VGPR-staged ring
     (3840, 3840, 128, GemmConfig(128, 128, 64, 64, 64, 1, 2, True, True, False, True)),  # tail
     (512, 512, 512, GemmConfig(256, 256, 64, 128, 128, 2, 1, False, False, False)),
@@ -124,6 +138,8 @@ GEMM_FULL = [
     (6144, 6144, 6144, GemmConfig(256, 256, 64, 128, 64, 2, 8, True, True, True, True)),
     (8192, 8192, 8192, GemmConfig(256, 256, 64, 128, 64, 2, 0, True, True, True, mfma=16, early=4)),
     (8192, 8192, 8192, GemmConfig(256, 256, 64, 128, 64, 2, 0, True, True, True, mfma=16, early=4, agpr=True)),
+    (8192, 8192, 8192, GemmConfig(256, 256, 64, 128, 64, 2, 0, True, True, True, mfma=16, early=4, agpr=True, spread=6)),
+    (6144, 6144, 6144, GemmConfig(256, 256, 64, 128, 64, 2, 0, True, True, True, True, mfma=16, agpr=True, spread=6)),
 ]
 
 
@@ -136,6 +152,7 @@ GEMM_BF16_CASES = [
     (512, 512, 512, GemmConfig(256, 256, 64, 128, 64, 2, 1, True, False, True, mfma=16, early=4)),
     (512, 1024, 256, GemmConfig(128, 128, 32, 64, 64, 3, 2, False, True, True, mfma=16)),
     (512, 512, 512, GemmConfig(256, 256, 64, 128, 64, 2, 1, True, False, True, mfma=16, agpr=True)),
+    (512, 1024, 256, GemmConfig(256, 256, 64, 128, 64, 2, 2, True, True, True, mfma=16, early=4, agpr=True, spread=6)),
 ]
 
 

@@ -335,3 +335,32 @@ def test_gemm_tail_split_is_offered_where_a_partial_wave_remains():
 
     plain = gm.GemmConfig(256, 256, 64, 128, 64, 2, 8, True, True, True)
     assert cm.gemm_tc_score(big, ARCH, 6144, 6144, 6144) > cm.gemm_tc_score(plain, ARCH, 6144, 6144, 6144)
+
+
+def test_gemm_spread_twins():
+    """Every 16x16x32 config whose K-tile has six or more MFMA groups comes with a twin whose
+    tile loads are dealt over the groups (`spread`); the 32x32x16 body has none."""
+    from deca_amd import tuned
+
+    cfgs = set(Solver.solve_gemm_tc(ARCH, 4096, 4096, 4096))
+    twins = [c for c in cfgs if c.spread]
+    assert twins and all(c.mfma == 16 and c.direct and replace(c, spread=0) in cfgs for c in twins)
+    assert all(c.spread == gm.default_spread(c) for c in twins)
+    assert all(replace(c, spread=gm.default_spread(c)) in cfgs
+               for c in cfgs if c.mfma == 16 and not c.spread and gm.default_spread(c))
+    big = gm.GemmConfig(256, 256, 64, 128, 64, 2, 0, True, True, True, mfma=16, early=4, agpr=True, spread=6)
+    assert big in cfgs and gm.mfma_groups_per_ktile(big) == 16 and gm.default_spread(big) == 6
+    small = gm.GemmConfig(128, 128, 64, 64, 32, 4, 4, True, True, True, mfma=16, early=2)
+    assert gm.mfma_groups_per_ktile(small) == 8 and gm.default_spread(small) == 3
+    assert gm.default_spread(gm.GemmConfig(64, 64, 32, 32, 64, 2, 2, False, False, True, mfma=16)) == 0
+    spec = gm.make_gemm_tc(4096, 4096, 4096, big)
+    defs, meta = dict(spec.defines), dict(spec.meta)
+    assert defs["DECA_DMA_SPREAD"] == 6 and defs["DECA_DMA_FIRST"] == gm.SPREAD_FIRST == 1
+    assert meta["no_scratch"] is True  # the prologue waits for part of its loads
+    plain = dict(gm.make_gemm_tc(4096, 4096, 4096, replace(big, spread=0)).defines)
+    assert "DECA_DMA_SPREAD" not in plain
+    assert str(big).endswith(",agpr=1,spread=6") and tuned.parse_config("GEMM", str(big)) == big
+    with pytest.raises(AssertionError):  # the 32x32x16 body issues its loads in one burst
+        gm.check_config(gm.GemmConfig(256, 256, 64, 128, 64, 2, 0, True, True, True, spread=6), 4096, 4096, 4096)
+    with pytest.raises(AssertionError):  # more groups than a K-tile has
+        gm.check_config(replace(big, spread=16), 4096, 4096, 4096)
