@@ -486,7 +486,7 @@ def solve_flash_attn(arch, B: int, H: int, S_q: int, S_kv: int, D: int, type_siz
         return []
     from dataclasses import replace
 
-    from deca_amd.kernels.flash_attn_hip import register_fill
+    from deca_amd.kernels.flash_attn_hip import default_spread, register_fill
 
     cons = _fa_constraints(arch, B, H, S_q, S_kv, D, type_size, max_est_regs)
     results = []
@@ -498,4 +498,7 @@ def solve_flash_attn(arch, B: int, H: int, S_q: int, S_kv: int, D: int, type_siz
         # run out of registers (it interacts with no other constraint: expanded here)
         if int(pipe) == 0 and st >= 2 and register_fill(cfg, D) >= 0.95:
             results.append(replace(cfg, roll=True))
+        # the next tile's loads dealt over the first matrix-instruction groups of a step
+        if default_spread(cfg):
+            results.append(replace(cfg, spread=default_spread(cfg)))
     return results

@@ -371,6 +371,10 @@ def fa_score(cfg, arch, shape, causal: bool = False) -> float:
     if cfg.stages == 3:
         tile_kib = cfg.Bc * D * 2 / 1024
         pipe *= 1.015 if tile_kib <= 8 else (0.98 if tile_kib <= 16 else 0.95)
+    # K/V loads dealt over the first groups of a step: +1 % in the slot loop, up to +3 % in the
+    # plain loop with short (64-key, D = 64) steps, nothing or a little less elsewhere
+    if getattr(cfg, "spread", 0):
+        pipe *= 1.01 if int(cfg.pipe) == 2 else (1.02 if cfg.Bc * D <= 64 * 64 else 0.995)
     if not getattr(cfg, "swizzle", True):
         pipe *= 0.5  # linear LDS rows: every fragment read is a multi-way bank conflict
     sync = 1.0 / (1.0 + getattr(arch, "fa_cta_sync_penalty", 0.0) * cfg.num_warps / 4 / wgs)

@@ -14,6 +14,9 @@
 //                       again from there in every KV step (flash_attn_tir.py:263-281,
 //                       345-348) instead of living in VGPRs for the whole kernel
 //   DECA_SWIZZLE        0: K/V/Q rows lie linearly in LDS (no XOR swizzle)
+//   DECA_SPREAD         n > 0: the K/V loads of the next tile are dealt over the first n
+//                       matrix-instruction groups of a step instead of issued in one burst
+//                       behind the barrier (two-stage plain and slot loops)
 //   DECA_CAUSAL         1: key j visible to query i iff j <= i (SQ == SKV)
 //   DECA_SCALE          softmax scale
 //   DECA_PIPE           1: S^T of the next tile is computed before the softmax of
@@ -79,6 +82,9 @@
 #endif
 #ifndef DECA_SWIZZLE
 #define DECA_SWIZZLE 1
+#endif
+#ifndef DECA_SPREAD
+#define DECA_SPREAD 0
 #endif
 #ifndef DECA_MIN_WAVES
 #define DECA_MIN_WAVES 1  // waves per SIMD the register allocation must leave room for
@@ -356,6 +362,26 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
     for (int it = 0; it < KV_IT; ++it) dma16(origin, v_voff[it], dst + it * NT * 16);
   };
 
+  // Load number l of the 2 * KV_IT that bring in tile j (K chunks first, then V), and the
+  // share of window position i out of n: all waves of a workgroup leave the step's barrier
+  // together, and issued in one burst their loads queue up at the CU's one load path (a
+  // 64-lane x 16-byte load per 16 clocks) while the waves in that queue issue nothing else.
+  auto issue_kv_load = [&](int jk, int kslot, int jv, int vslot, int l) __attribute__((always_inline)) {
+    if (l < KV_IT) {
+      if (jk < nkv)
+        dma16(k_base + static_cast<size_t>(jk) * BC * D_, k_voff[l],
+              lds_u + kslot * TILE_BYTES + wave_u * 1024 + l * NT * 16);
+    } else {
+      dma16(v_base + static_cast<size_t>(jv) * BC * D_, v_voff[l - KV_IT],
+            lds_u + (STAGES + vslot) * TILE_BYTES + wave_u * 1024 + (l - KV_IT) * NT * 16);
+    }
+  };
+  auto issue_kv_share = [&](int jk, int kslot, int jv, int vslot, int i, int n) __attribute__((always_inline)) {
+#pragma unroll
+    for (int l = i * (2 * KV_IT) / n; l < (i + 1) * (2 * KV_IT) / n; ++l)
+      issue_kv_load(jk, kslot, jv, vslot, l);
+  };
+
   // ---- Q fragments: VGPR resident for the whole kernel ----------------------------
   // lane (q = lane % 32, half): 8 consecutive d at ks * 16 + half * 8
   // (16x16x32: q = lane % 16, 8 consecutive d at ks * 32 + (lane / 16) * 8)
@@ -447,7 +473,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
   };
   // ---- the three phases of one KV step ----------------------------------------------------
   // S^T = K Q^T for the tile in K slot `kslot`
-  auto compute_s = [&](acc_t (&s_acc)[KT][MQ], int kslot) __attribute__((always_inline)) {
+  auto compute_s = [&](acc_t (&s_acc)[KT][MQ], int kslot, auto&& between) __attribute__((always_inline)) {
     const unsigned char* k_lds = lds + kslot * TILE_BYTES;
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt)
@@ -466,9 +492,11 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
 #pragma unroll
         for (int mq = 0; mq < MQ; ++mq)
           s_acc[kt][mq] = DECA_MFMA(kf, qk[mq], s_acc[kt][mq], 0, 0, 0);
+        between(ks * KT + kt);
       }
     }
   };
+  auto nothing = [](int) __attribute__((always_inline)) {};
   // Causal mask of tile j.  Only tiles crossing the diagonal need it; every
   // query sees key 0 in tile 0, so its running max is finite before a fully
   // masked block shows up.
@@ -628,7 +656,14 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
     // Tile j has landed for every lane, and every wave is done with the slot
     // that tile j+1 is about to overwrite.
     wait_and_barrier();
-    if (j + 1 < nkv) {
+    constexpr int SPREAD_N = DECA_SPREAD < DK * KT ? DECA_SPREAD : DK * KT;
+    const bool more = j + 1 < nkv;
+#if DECA_CAUSAL
+    const bool skip = j * BC > qt * BR + wave_u * WQ + WQ - 1;
+#else
+    const bool skip = false;
+#endif
+    if (more && (SPREAD_N == 0 || skip)) {
       issue_k(j + 1, slot ^ 1);
       issue_v(j + 1, slot ^ 1);
     }
@@ -643,7 +678,14 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
 #endif
     acc_t s_acc[KT][MQ];
     half8 pf[KK][MQ];
-    compute_s(s_acc, slot);
+#if STAGES == 2 && DECA_SPREAD > 0
+    // the next tile's loads ride on the first SPREAD_N groups of S^T instructions
+    compute_s(s_acc, slot, [&](int i) __attribute__((always_inline)) {
+      if (i < SPREAD_N && more) issue_kv_share(j + 1, slot ^ 1, j + 1, slot ^ 1, i, SPREAD_N);
+    });
+#else
+    compute_s(s_acc, slot, nothing);
+#endif
     mask_s(s_acc, j);
     softmax(s_acc, pf);
     compute_pv(pf, slot);
@@ -817,7 +859,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
   };
   half2v pf2[KK][MQ][4];
   // Score number n of a lane and query tile lives in accumulator n / ACC_N, register n % ACC_N.
-  auto fused = [&](auto v_slot, acc_t (&sc)[KT][MQ], acc_t (&sn)[KT][MQ]) __attribute__((always_inline)) {
+  auto fused = [&](auto v_slot, acc_t (&sc)[KT][MQ], acc_t (&sn)[KT][MQ], int j) __attribute__((always_inline)) {
     constexpr int VSLOT = decltype(v_slot)::value;  // V_j; K_{j+1} is in the other K slot
     const unsigned char* k_lds = lds + (VSLOT ^ 1) * TILE_BYTES;
     const unsigned char* v_lds = lds + (STAGES + VSLOT) * TILE_BYTES;
@@ -896,6 +938,9 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
     static_for<NS>([&](auto tc) {
       constexpr int t = decltype(tc)::value;
       if constexpr (t + 2 < NS) frag[(t + 2) % 3] = read_frag(std::integral_constant<int, t + 2>{});
+      // K_{j+2} and V_{j+1} go where K_j and V_{j-1} were: their loads ride on the first slots
+      constexpr int SPREAD_S = DECA_SPREAD < NS ? DECA_SPREAD : NS;
+      if constexpr (t < SPREAD_S) issue_kv_share(j + 2, VSLOT, j + 1, VSLOT ^ 1, t, SPREAD_S);
       if constexpr (t < S_SLOTS) {
         constexpr int pr = t / (2 * DK), r = t % (2 * DK), ks = r / 2, kt = 2 * pr + r % 2;
         static_for<MQ>([&](auto mqc) {
@@ -924,12 +969,14 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
   auto step = [&](auto cur_slot, acc_t (&sc)[KT][MQ], acc_t (&sn)[KT][MQ], int j) __attribute__((always_inline)) {
     constexpr int cur = decltype(cur_slot)::value;  // == j % 2
     wait_and_barrier();  // K_{j+1}, V_j landed; everyone is done with K_j and V_{j-1}
+#if DECA_SPREAD == 0
     if (j + 2 < nkv) issue_k(j + 2, cur);
     issue_v(j + 1, cur ^ 1);
+#endif
     // The O^T rescale stays out of the slots: with the lazy running max it is needed
     // for the first tile and then hardly ever, so it is a branch of its own here.
     rescale_o();
-    fused(cur_slot, sc, sn);
+    fused(cur_slot, sc, sn, j);
   };
   auto tail = [&](acc_t (&sc)[KT][MQ], int j) __attribute__((always_inline)) {
     wait_and_barrier();
@@ -957,7 +1004,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
     issue_k(1, 1);
     acc_t s_a[KT][MQ], s_b[KT][MQ];
     wait_and_barrier();
-    compute_s(s_a, 0);
+    compute_s(s_a, 0, nothing);
     row_stats(s_a);
     int j = 0;
     for (; j + 2 < nd; j += 2) {
@@ -986,7 +1033,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
   if (nkv > 1) issue_k(1, 1);
   acc_t s_a[KT][MQ], s_b[KT][MQ];
   wait_and_barrier();
-  compute_s(s_a, 0);
+  compute_s(s_a, 0, nothing);
   row_stats(s_a);
   {
     int j = 0;
@@ -1009,7 +1056,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
   floatx16 s_cur[KT][MQ], s_nxt[KT][MQ];
   half8 pf[KK][MQ];
   wait_and_barrier();
-  compute_s(s_cur, 0);
+  compute_s(s_cur, 0, nothing);
   mask_s(s_cur, 0);
   row_stats(s_cur);
   for (int j = 0; j < nkv - 1; ++j) {
@@ -1072,7 +1119,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
     wait_and_barrier();
     acc_t s_acc[KT][MQ];
     half8 pf[KK][MQ];
-    compute_s(s_acc, 0);
+    compute_s(s_acc, 0, nothing);
     mask_s(s_acc, j);
     softmax(s_acc, pf);
     compute_pv(pf, 0);

@@ -55,6 +55,12 @@ class FAConfig:
     # True keeps one copy with the slot as a run-time value (about 50 registers fewer: for
     # the tiles whose unrolled loop does not fit the register file of two waves per SIMD).
     roll: bool = False
+    # Two-stage plain loop and slot loop: the K/V loads of the next tile are dealt over the
+    # first `spread` groups of matrix instructions of a step instead of issued in one burst
+    # behind the step's barrier, where all waves queue up at the CU's one load path
+    # (measured: +1 % for the D = 128 slot loop with 8, +3 % for the D = 64 plain loop with 2-4,
+    # -1...-2 % for the rolled 16x16x32 loop).
+    spread: int = 0
 
     @property
     def threads(self) -> int:
@@ -70,7 +76,16 @@ class FAConfig:
             + (f",pipe={int(self.pipe)}" if self.pipe else "")
             + (f",mfma={self.mfma}" if self.mfma != 32 else "")
             + (",roll=1" if self.roll else "")
+            + (f",spread={self.spread}" if self.spread else "")
         )
+
+
+def default_spread(cfg: FAConfig) -> int:
+    """The window the solver offers: 8 slots in the slot loop, 4 groups in the unrolled
+    two-stage plain loop, none elsewhere."""
+    if cfg.stages != 2 or cfg.roll:
+        return 0
+    return 8 if int(cfg.pipe) == 2 else (4 if int(cfg.pipe) == 0 else 0)
 
 
 def smem_bytes(cfg: FAConfig, D: int) -> int:
@@ -175,6 +190,9 @@ def check_config(cfg: FAConfig, S_q: int, S_kv: int, D: int) -> None:
     assert cfg.mfma == 32 or int(cfg.pipe) != 1, "the 16x16x32 form exists for the plain and the slot loop"
     assert not cfg.pipe or cfg.stages == 2
     assert not cfg.roll or (int(cfg.pipe) == 0 and cfg.stages >= 2), "roll is a form of the plain ring loop"
+    assert cfg.spread >= 0
+    assert not cfg.spread or (cfg.stages == 2 and int(cfg.pipe) in (0, 2)), \
+        "the load window exists in the two-stage plain and slot loops"
     assert int(cfg.pipe) != 2 or slot_schedule_ok(cfg.Bc, D, cfg.mfma)
     # a wave's Q rows go to LDS as whole 1 KiB runs
     assert not cfg.q_in_smem or (cfg.Br // cfg.num_warps * cpr) % WAVE == 0
@@ -215,6 +233,8 @@ def make_flash_attn_fwd(
         defines["DECA_QSMEM"] = 1
     if not cfg.swizzle:
         defines["DECA_SWIZZLE"] = 0
+    if cfg.spread:
+        defines["DECA_SPREAD"] = cfg.spread
     # The three-stage ring waits for part of its outstanding loads, which is only right
     # while the tile loads are the loop's only vector-memory traffic: a build that spills
     # (scratch stores share the counter and retire out of order) is refused at load time.

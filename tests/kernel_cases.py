@@ -249,6 +249,16 @@ FA_CASES = [
     (2, 2, 512, 512, 64, True, FAConfig(256, 64, 4, 3, mfma=16, roll=True)),
     (1, 2, 256, 320, 128, False, FAConfig(128, 64, 4, 3, roll=True)),
     (1, 2, 512, 512, 192, True, FAConfig(128, 32, 4, 3, q_in_smem=True, mfma=16)),
+    # the next tile's loads dealt over the first groups of a step: plain and slot loop, both
+    # tile forms, full and causal (masked tiles skipped by some waves), odd numbers of tiles
+    (1, 2, 512, 512, 128, False, FAConfig(256, 64, 8, 2, pipe=2, spread=8)),
+    (1, 2, 512, 512, 128, True, FAConfig(256, 64, 8, 2, pipe=2, mfma=16, spread=4)),
+    (2, 2, 512, 512, 64, True, FAConfig(256, 128, 8, 2, pipe=2, spread=8)),
+    (1, 2, 256, 384, 128, False, FAConfig(128, 128, 4, 2, pipe=2, spread=100)),
+    (2, 2, 512, 512, 64, False, FAConfig(256, 64, 4, 2, spread=4)),
+    (1, 2, 512, 512, 128, True, FAConfig(256, 64, 8, 2, mfma=16, spread=2)),
+    (1, 2, 256, 320, 64, False, FAConfig(128, 64, 4, 2, spread=1)),
+    (1, 2, 512, 512, 64, True, FAConfig(128, 128, 4, 2, q_in_smem=True, spread=4)),
     # linear LDS rows (no swizzle): both row lengths, both tile forms, with and without the
     # staged Q tile
     (1, 2, 256, 256, 128, True, FAConfig(128, 64, 4, 2, swizzle=False)),
@@ -268,6 +278,8 @@ FA_FULL = [
     (4, 16, 4096, 4096, 128, True, FAConfig(256, 64, 8, 2, pipe=2)),
     (4, 16, 4096, 4096, 128, False, FAConfig(256, 64, 8, 2, q_in_smem=True, mfma=16)),
     (4, 16, 4096, 4096, 64, True, FAConfig(256, 64, 4, 3, q_in_smem=True)),
+    (4, 16, 4096, 4096, 128, True, FAConfig(256, 64, 8, 2, pipe=2, spread=8)),
+    (4, 16, 4096, 4096, 64, False, FAConfig(256, 64, 4, 2, spread=4)),
 ]
 
 

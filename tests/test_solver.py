@@ -157,6 +157,9 @@ def test_flash_attn_configs_are_valid(D, S):
         # the one-copy form of the plain ring loop, where the unrolled one is tight
         if pipe == 0 and st >= 2 and fa.register_fill(cfg, D) >= 0.95:
             want.add(replace(cfg, roll=True))
+        # the load window of the two-stage plain and slot loops
+        if st == 2 and pipe in (0, 2):
+            want.add(replace(cfg, spread=8 if pipe == 2 else 4))
     assert set(configs) == want
     # the reference's knobs are all in the search (Solver.py:330-336), except linear LDS rows
     assert {c.stages for c in configs} == {1, 2, 3}
@@ -274,6 +277,15 @@ def test_flash_attn_knobs_of_the_reference():
     # the winner tile of D = 128 (a 128 KiB ring) has no room for a 64 KiB Q tile
     with pytest.raises(AssertionError):
         fa.check_config(fa.FAConfig(256, 128, 8, 2, q_in_smem=True), 4096, 4096, 128)
+    # the spread load window: two-stage plain and slot loops only
+    assert fa.default_spread(base) == 4 and fa.default_spread(replace(base, pipe=2)) == 8
+    assert fa.default_spread(deep) == 0 and fa.default_spread(replace(base, roll=True)) == 0
+    sp = replace(base, pipe=2, spread=8)
+    assert dict(fa.make_flash_attn_fwd(4, 16, 4096, 4096, 128, sp).defines)["DECA_SPREAD"] == 8
+    assert str(sp).endswith(",pipe=2,spread=8")
+    for bad in (replace(deep, spread=4), replace(base, pipe=1, spread=4), replace(base, stages=1, spread=4)):
+        with pytest.raises(AssertionError):
+            fa.check_config(bad, 4096, 4096, 128)
     # three stages belong to the plain loop; four do not exist
     for bad in (fa.FAConfig(128, 64, 4, 3, pipe=2), fa.FAConfig(128, 64, 4, 3, pipe=1), fa.FAConfig(128, 64, 4, 4)):
         with pytest.raises(AssertionError):
