@@ -194,7 +194,7 @@ def summary_text(workload: str, out_dir: str, kernel_config: str | None = None) 
     write = counter_means(_rows(os.path.join(out_dir, "write", "out_counter_collection.csv")))
 
     def rel(cmd):
-        words = [f"'{w}'" if "," in w else w for w in cmd]
+        words = [f"'{w}'" if ("," in w or not w) else w for w in cmd]
         return " ".join(words).replace(ROOT + os.sep, "").replace(out_dir, "<out>")
 
     extra = f" --kernel-config '{kernel_config}'" if kernel_config else ""
