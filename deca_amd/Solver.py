@@ -380,7 +380,7 @@ def solve_gemm_tc(arch, M: int, N: int, K: int, type_size: int = 2, count: int =
                 if default_spread(cfg):
                     cands += [replace(c, spread=default_spread(cfg)) for c in cands]
             for cand in cands:
-                if ras == 0 or cand.tail:
+                if ras == 0 or cand.tail or cand.spread:
                     try:
                         check_config(cand, M, N, K)
                     except AssertionError:

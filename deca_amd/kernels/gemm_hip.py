@@ -110,9 +110,32 @@ def mfma_groups_per_ktile(cfg: GemmConfig) -> int:
     return (cfg.BK // 32) * (cfg.warp_m // 16)
 
 
+def spread_head_loads(loads: int, mt: int, ks: int, early: int, spread: int) -> int:
+    """Loads of the second tile that the prologue issues with `spread` (what the groups
+    behind a barrier would have issued of it), as the kernel computes it: the window has
+    `ks * mt` groups, the first `mt - early` of them lie behind the barrier, and the loads
+    are dealt over `spread` groups starting `SPREAD_FIRST` groups in."""
+    if not spread:
+        return 0
+    groups = ks * mt
+    early = min(early, mt - 1)
+    post = mt - early
+    n = min(spread, groups)
+    first = SPREAD_FIRST if SPREAD_FIRST + n <= groups else groups - n
+    if post <= first:
+        return 0
+    return loads if post - first >= n else (post - first) * loads // n
+
+
 def default_spread(cfg: GemmConfig) -> int:
     """The window the solver offers for a tile: 6 groups where a K-tile has 12 or more
-    (measured best of 2..12 for 256 x 256 x 64 tiles), 3 where it has 6 or more, else none."""
+    (measured best of 2..12 for 256 x 256 x 64 tiles), 3 where it has 6 or more, else none --
+    and none where the register estimate fills the budget of the waves that share a SIMD to
+    the last eight registers: such a build spills a few registers (64 x 128 wave tiles of the
+    builtin 16x16x32 body: 8-44 bytes), and with the load window's partial wait in the
+    prologue the loader refuses a build that spills."""
+    if (est_regs_per_thread(cfg) + 8) * -(-cfg.num_warps // 4) > MAX_VGPRS:
+        return 0
     groups = mfma_groups_per_ktile(cfg)
     return 6 if groups >= 12 else (3 if groups >= 6 else 0)
 
@@ -231,9 +254,11 @@ def check_config(cfg: GemmConfig, M: int, N: int, K: int, max_smem: int = MAX_LD
     assert (cfg.BM * cfg.BK // 8) % cfg.threads == 0
     assert (cfg.BK * cfg.BN // 8) % cfg.threads == 0
     if cfg.direct:
-        # loads left in flight by the (stages - 2) youngest tiles fit the 6-bit counter
+        # loads left in flight by the (stages - 2) youngest tiles -- and, with `spread`, the
+        # head of the next one in the prologue -- fit the 6-bit counter
         loads = (cfg.BM * cfg.BK + cfg.BK * cfg.BN) // 8 // cfg.threads
-        assert (cfg.stages - 2) * loads <= 63
+        head = spread_head_loads(loads, cfg.warp_m // 16, cfg.BK // 32, cfg.early, cfg.spread)
+        assert (cfg.stages - 2) * loads + head <= 63
     if cfg.tail:
         r = tail_tiles(cfg, M, N)
         tiles = (M // cfg.BM) * (N // cfg.BN)
@@ -247,7 +272,8 @@ def check_config(cfg: GemmConfig, M: int, N: int, K: int, max_smem: int = MAX_LD
         assert K // cfg.BK >= qs
         if cfg.direct:
             q_loads = (cfg.BM // 2 * cfg.BK + cfg.BK * (cfg.BN // 2)) // 8 // cfg.threads
-            assert (qs - 2) * q_loads <= 63
+            q_head = spread_head_loads(q_loads, max(1, cfg.warp_m // 32), cfg.BK // 32, cfg.early, cfg.spread)
+            assert (qs - 2) * q_loads + q_head <= 63
     if cfg.raster == 0:
         full = (M // cfg.BM) * (N // cfg.BN) - (tail_tiles(cfg, M, N) if cfg.tail else 0)
         assert cfg.xcd and (M // cfg.BM) % 8 == 0 and (N // cfg.BN) % 4 == 0 and full % 256 == 0

@@ -358,8 +358,17 @@ def test_gemm_spread_twins():
     twins = [c for c in cfgs if c.spread]
     assert twins and all(c.mfma == 16 and c.direct and replace(c, spread=0) in cfgs for c in twins)
     assert all(c.spread == gm.default_spread(c) for c in twins)
-    assert all(replace(c, spread=gm.default_spread(c)) in cfgs
-               for c in cfgs if c.mfma == 16 and not c.spread and gm.default_spread(c))
+    def valid(c):
+        try:
+            gm.check_config(c, 4096, 4096, 4096)
+            return True
+        except AssertionError:
+            return False
+
+    for c in cfgs:
+        if c.mfma == 16 and not c.spread and gm.default_spread(c):
+            twin = replace(c, spread=gm.default_spread(c))
+            assert (twin in cfgs) == valid(twin), c
     big = gm.GemmConfig(256, 256, 64, 128, 64, 2, 0, True, True, True, mfma=16, early=4, agpr=True, spread=6)
     assert big in cfgs and gm.mfma_groups_per_ktile(big) == 16 and gm.default_spread(big) == 6
     small = gm.GemmConfig(128, 128, 64, 64, 32, 4, 4, True, True, True, mfma=16, early=2)
@@ -376,3 +385,23 @@ def test_gemm_spread_twins():
         gm.check_config(gm.GemmConfig(256, 256, 64, 128, 64, 2, 0, True, True, True, spread=6), 4096, 4096, 4096)
     with pytest.raises(AssertionError):  # more groups than a K-tile has
         gm.check_config(replace(big, spread=16), 4096, 4096, 4096)
+
+
+def test_gemm_spread_prologue_fits_the_load_counter():
+    """With `spread` the prologue leaves the head of the second tile in flight beside the
+    (stages - 2) youngest tiles; the host mirrors the kernel's count, and the solver drops the
+    deep one-wave rings where the 6-bit counter would overflow."""
+    assert gm.spread_head_loads(8, 8, 2, 4, 6) == 4      # 256 x 256 x 64, 8 waves: half a tile
+    assert gm.spread_head_loads(8, 8, 2, 4, 0) == 0
+    assert gm.spread_head_loads(16, 4, 2, 0, 3) == 16    # window shorter than the groups behind the barrier
+    deep = gm.GemmConfig(64, 64, 64, 64, 64, 5, 1, True, True, True, mfma=16, agpr=True, spread=3)
+    with pytest.raises(AssertionError):
+        gm.check_config(deep, 2048, 2048, 2048)          # 3 x 16 + 16 loads in flight
+    gm.check_config(replace(deep, spread=0), 2048, 2048, 2048)
+    cfgs = Solver.solve_gemm_tc(ARCH, 2048, 2048, 2048)
+    assert deep not in cfgs and replace(deep, spread=0) in cfgs
+    for c in cfgs:
+        if c.spread:
+            loads = (c.BM * c.BK + c.BK * c.BN) // 8 // c.threads
+            head = gm.spread_head_loads(loads, c.warp_m // 16, c.BK // 32, c.early, c.spread)
+            assert (c.stages - 2) * loads + head <= 63
