@@ -408,7 +408,7 @@ def main():
     ap.add_argument("--power", type=int, default=0, metavar="SECONDS",
                     help="after timing a workload, sample shader clock and socket power once a "
                          "second for this long while its kernel repeats (roofline.sclk_mhz / socket_w)")
-    ap.add_argument("--full-out", default=os.path.join(ROOT, "gpurun_out", "bench_full.json"),
+    ap.add_argument("--full-out", default=os.path.join(ROOT, "bench_full.json"),
                     metavar="PATH", help="file for the full per-workload records ('' for none)")
     args = ap.parse_args()
     if args.gpus != 1:

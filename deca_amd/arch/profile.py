@@ -195,7 +195,7 @@ def summary_text(workload: str, out_dir: str, kernel_config: str | None = None) 
 
     def rel(cmd):
         words = [f"'{w}'" if ("," in w or not w) else w for w in cmd]
-        return " ".join(words).replace(ROOT + os.sep, "").replace(out_dir, "<out>")
+        return " ".join(words).replace(out_dir, "<out>").replace(ROOT + os.sep, "")
 
     extra = f" --kernel-config '{kernel_config}'" if kernel_config else ""
     t = [f"# rocprofv3 summary: `{kern}.hip` on workload `{workload}`"
@@ -305,13 +305,13 @@ def main(argv=None):
     ap.add_argument("action", choices=["run", "summarise"])
     ap.add_argument("workload")
     ap.add_argument("--out", default=None, help="directory of the passes' output "
-                                                "(default gpurun_out/prof_<workload>[_<tag>])")
+                                                "(default profile_out/prof_<workload>[_<tag>])")
     ap.add_argument("--kernel-config", default=None, metavar="TEXT",
                     help="profile this configuration instead of the stored winner")
     ap.add_argument("--tag", default="variant", help="with --kernel-config: suffix of the summary's name")
     args = ap.parse_args(argv)
     default = f"prof_{args.workload}" + (f"_{args.tag}" if args.kernel_config else "")
-    out_dir = os.path.abspath(args.out or os.path.join(ROOT, "gpurun_out", default))
+    out_dir = os.path.abspath(args.out or os.path.join(ROOT, "profile_out", default))
     if args.action == "run":
         run(args.workload, out_dir, kernel_config=args.kernel_config)
     else:
