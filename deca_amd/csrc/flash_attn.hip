@@ -16,7 +16,7 @@
 //   DECA_SWIZZLE        0: K/V/Q rows lie linearly in LDS (no XOR swizzle)
 //   DECA_SPREAD         n > 0: the K/V loads of the next tile are dealt over the first n
 //                       matrix-instruction groups of a step instead of issued in one burst
-//                       behind the barrier (two-stage plain and slot loops)
+//                       behind the barrier (plain ring loops and slot loop)
 //   DECA_CAUSAL         1: key j visible to query i iff j <= i (SQ == SKV)
 //   DECA_SCALE          softmax scale
 //   DECA_PIPE           1: S^T of the next tile is computed before the softmax of
@@ -647,41 +647,39 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
     __builtin_amdgcn_s_waitcnt(0xC07F);
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    if (j + 2 < nkv) {
-      const int fill = slot == 0 ? 2 : slot - 1;
-      issue_k(j + 2, fill);
-      issue_v(j + 2, fill);
-    }
+    const int ahead = j + 2;                        // the tile this step requests ...
+    const int fill = slot == 0 ? 2 : slot - 1;      // ... and the ring slot it goes to
 #else
     // Tile j has landed for every lane, and every wave is done with the slot
     // that tile j+1 is about to overwrite.
     wait_and_barrier();
+    const int ahead = j + 1;
+    const int fill = slot ^ 1;
+#endif
     constexpr int SPREAD_N = DECA_SPREAD < DK * KT ? DECA_SPREAD : DK * KT;
-    const bool more = j + 1 < nkv;
-#if DECA_CAUSAL
-    const bool skip = j * BC > qt * BR + wave_u * WQ + WQ - 1;
-#else
-    const bool skip = false;
-#endif
-    if (more && (SPREAD_N == 0 || skip)) {
-      issue_k(j + 1, slot ^ 1);
-      issue_v(j + 1, slot ^ 1);
-    }
-#endif
+    const bool more = ahead < nkv;
 #if DECA_CAUSAL
     // Every key of the tile lies after every query row of this wave (the last tile
     // of a workgroup with BR > BC): all its scores are masked, P = 0 exactly, and
     // there is nothing to add.  (Skipping single masked 32-key blocks of the
     // diagonal tiles as well was tried: the extra code paths cost registers and
     // made the kernel slower.)
-    if (j * BC > qt * BR + wave_u * WQ + WQ - 1) return;
+    const bool skip = j * BC > qt * BR + wave_u * WQ + WQ - 1;
+#else
+    const bool skip = false;
 #endif
+    // one burst behind the barrier, or (DECA_SPREAD) dealt over the S^T groups below
+    if (more && (SPREAD_N == 0 || skip)) {
+      issue_k(ahead, fill);
+      issue_v(ahead, fill);
+    }
+    if (skip) return;
     acc_t s_acc[KT][MQ];
     half8 pf[KK][MQ];
-#if STAGES == 2 && DECA_SPREAD > 0
-    // the next tile's loads ride on the first SPREAD_N groups of S^T instructions
+#if DECA_SPREAD > 0
+    // the requested tile's loads ride on the first SPREAD_N groups of S^T instructions
     compute_s(s_acc, slot, [&](int i) __attribute__((always_inline)) {
-      if (i < SPREAD_N && more) issue_kv_share(j + 1, slot ^ 1, j + 1, slot ^ 1, i, SPREAD_N);
+      if (i < SPREAD_N && more) issue_kv_share(ahead, fill, ahead, fill, i, SPREAD_N);
     });
 #else
     compute_s(s_acc, slot, nothing);

@@ -259,6 +259,9 @@ FA_CASES = [
     (1, 2, 512, 512, 128, True, FAConfig(256, 64, 8, 2, mfma=16, spread=2)),
     (1, 2, 256, 320, 64, False, FAConfig(128, 64, 4, 2, spread=1)),
     (1, 2, 512, 512, 64, True, FAConfig(128, 128, 4, 2, q_in_smem=True, spread=4)),
+    (2, 2, 512, 512, 64, False, FAConfig(256, 64, 4, 3, spread=4)),
+    (1, 2, 512, 512, 128, True, FAConfig(128, 64, 4, 3, mfma=16, spread=2)),
+    (1, 2, 256, 320, 64, False, FAConfig(128, 64, 2, 3, spread=100)),
     # linear LDS rows (no swizzle): both row lengths, both tile forms, with and without the
     # staged Q tile
     (1, 2, 256, 256, 128, True, FAConfig(128, 64, 4, 2, swizzle=False)),

@@ -280,10 +280,11 @@ def test_flash_attn_knobs_of_the_reference():
     # the spread load window: two-stage plain and slot loops only
     assert fa.default_spread(base) == 4 and fa.default_spread(replace(base, pipe=2)) == 8
     assert fa.default_spread(deep) == 0 and fa.default_spread(replace(base, roll=True)) == 0
+    fa.check_config(replace(deep, spread=4), 4096, 4096, 128)  # accepted, just not offered
     sp = replace(base, pipe=2, spread=8)
     assert dict(fa.make_flash_attn_fwd(4, 16, 4096, 4096, 128, sp).defines)["DECA_SPREAD"] == 8
     assert str(sp).endswith(",pipe=2,spread=8")
-    for bad in (replace(deep, spread=4), replace(base, pipe=1, spread=4), replace(base, stages=1, spread=4)):
+    for bad in (replace(base, pipe=1, spread=4), replace(base, stages=1, spread=4)):
         with pytest.raises(AssertionError):
             fa.check_config(bad, 4096, 4096, 128)
     # three stages belong to the plain loop; four do not exist
