@@ -83,7 +83,7 @@ def _board(kern, sets):
     from deca_amd.arch import ceilings
 
     buf = io.StringIO()
-    ceilings._sample_while(lambda: [kern(*sets[i % len(sets)]) for i in range(50)], "board", buf,
+    ceilings.sample_while(lambda: [kern(*sets[i % len(sets)]) for i in range(50)], "board", buf,
                            seconds=POWER_SECONDS + 1)
     lines = buf.getvalue().splitlines()[1:]  # the first second still ramps
     for line in lines:

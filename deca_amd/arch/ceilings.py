@@ -212,7 +212,7 @@ def measure_mfma(out=sys.stdout):
                   f"{flops / t / 1e12:6.0f} TFLOP/s ({t * 1e3:.3f} ms)", file=out, flush=True)
 
 
-def _board_state():
+def board_state():
     """Shader clock, socket power and power cap as rocm-smi reports them, on one line."""
     try:
         text = subprocess.run(["rocm-smi", "--showclocks", "--showpower", "--showmaxpower"],
@@ -229,7 +229,7 @@ def _board_state():
     return " | ".join(keep)
 
 
-def _sample_while(launch, label, out, seconds=3):
+def sample_while(launch, label, out, seconds=3):
     """Prints the board state once a second while `launch()` (a batch of asynchronous
     launches) repeats on a worker thread."""
     import torch
@@ -245,7 +245,7 @@ def _sample_while(launch, label, out, seconds=3):
     worker.start()
     for _ in range(seconds):
         time.sleep(1.0)
-        print(f"{label}: {_board_state()}", file=out, flush=True)
+        print(f"{label}: {board_state()}", file=out, flush=True)
     stop.set()
     worker.join()
 
@@ -264,13 +264,13 @@ def measure_sclk(out=sys.stdout):
     n = 8192
     cfg = tuned.lookup(tuned.make_key("GEMM", (n, n, n), "float16", "gfx950", False, "uniform"))
     kern = build_gemm_tc(make_gemm_tc(n, n, n, cfg))
-    print(f"idle: {_board_state()}", file=out, flush=True)
+    print(f"idle: {board_state()}", file=out, flush=True)
     makers = {"U(-1,1)": lambda: (2 * torch.rand(n, n, device="cuda") - 1).half(),
               "zeros": lambda: torch.zeros(n, n, device="cuda", dtype=torch.float16)}
     for name, make in makers.items():
         a, b = make(), make()
         c = torch.empty(n, n, device="cuda", dtype=torch.float16)
-        _sample_while(lambda: [kern(a, b, c) for _ in range(50)], f"GEMM {n}^3 [{cfg}] on {name}", out)
+        sample_while(lambda: [kern(a, b, c) for _ in range(50)], f"GEMM {n}^3 [{cfg}] on {name}", out)
         t = kern.time([(a, b, c)], 20)
         print(f"  -> {2 * n**3 / t / 1e12:.0f} TFLOP/s", file=out, flush=True)
     for d in (128, 64):
@@ -279,14 +279,14 @@ def measure_sclk(out=sys.stdout):
         fa = build_flash_attn(make_flash_attn_fwd(*shape, fcfg, None, False))
         q, k, v = make_qkv(*shape)
         o = torch.empty_like(q)
-        _sample_while(lambda: [fa(q, k, v, o) for _ in range(50)], f"FlashAttention D{d} [{fcfg}] on N(0,1)", out)
+        sample_while(lambda: [fa(q, k, v, o) for _ in range(50)], f"FlashAttention D{d} [{fcfg}] on N(0,1)", out)
         t = fa.time([(q, k, v, o)], 20)
         print(f"  -> {attn_flops(*shape, False) / t / 1e12:.0f} TFLOP/s", file=out, flush=True)
     spec = mfma_spec(3, 8, 2048)
     loop = load_kernel(spec, cached_build(spec))
     x = torch.randn(4096 * 8, device="cuda").half()
     res = torch.empty(2048 * 256, device="cuda")
-    _sample_while(lambda: [loop(x, res) for _ in range(10)], "MFMA 32x32x16 register-only loop on N(0,1)", out)
+    sample_while(lambda: [loop(x, res) for _ in range(10)], "MFMA 32x32x16 register-only loop on N(0,1)", out)
 
 
 def main(argv=None):
