@@ -2,8 +2,9 @@
 Loads, verifies and times one tuned kernel.
 
 Same constructor, methods and result attributes as the reference's
-src/RuntimeMod.py (`build`, `load_kernel`, `load_flash_attn`, `time_evaluator`,
-`time_kernel_op`, `time_flash_attn`, `show`, `get_mod`; `execution_time`,
+src/RuntimeMod.py (`build`, `build_with_tc`, `build_flash_attn`, `load_kernel`,
+`load_flash_attn`, `time_evaluator`, `time_kernel_op`, `time_flash_attn`, `show`,
+`get_mod`, `get_sch`; `execution_time`,
 `throughput`, `max_error`, `record`).  Underneath, a kernel is a gfx950 code
 object loaded through libdeca_hip.so instead of a TVM runtime module, and torch
 tensors are handed over as raw device pointers instead of DLPack capsules.
@@ -71,6 +72,12 @@ class RuntimeMod:
         self.runtime_mod = self.operator.compile(self._specialise())
 
     build_flash_attn = build
+    build_with_tc = build  # every GEMM here is a config-generated MFMA kernel (RuntimeMod.py:79-87)
+
+    def build_without_tc(self):
+        """The reference's CUDA-core GEMM over a TVM schedule (RuntimeMod.py:67-77) has no
+        counterpart here: the operators of this build all generate their kernel from a config."""
+        raise NotImplementedError("no schedule-based GEMM in this build: use the GEMMTC operator")
 
     def load_kernel(self, path: str):
         """Load a code object written by one of the `build_*_to_file` functions."""
@@ -82,6 +89,12 @@ class RuntimeMod:
 
     def get_mod(self):
         return self.ir_mod
+
+    def get_sch(self):
+        """The TVM schedule of the reference's legacy GEMM path (RuntimeMod.py:126-131); never
+        built here, so this fails the way the reference does before its `build_*_tc`."""
+        assert hasattr(self, "sch"), "Schedule not built"
+        return self.sch
 
     def show(self):
         """Print the specialisation (template, macros, geometry) and, once

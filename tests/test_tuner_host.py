@@ -181,6 +181,14 @@ def test_runtime_mod_error_metric_and_nan():
     with pytest.raises(RuntimeError, match="no kernel loaded"):
         rt.time_kernel_op()
     assert rt.is_flash_attn is False
+    # the reference's method names (RuntimeMod.py:53-131): the tensor-core build is the build,
+    # its schedule-based legacy path says what it is not
+    assert RuntimeMod.build_with_tc is RuntimeMod.build and RuntimeMod.build_flash_attn is RuntimeMod.build
+    assert RuntimeMod.load_flash_attn is RuntimeMod.load_kernel
+    with pytest.raises(NotImplementedError, match="GEMMTC"):
+        rt.build_without_tc()
+    with pytest.raises(AssertionError, match="Schedule not built"):
+        rt.get_sch()
 
 
 def test_tuned_table_roundtrip(tmp_path):
