@@ -493,12 +493,17 @@ def solve_flash_attn(arch, B: int, H: int, S_q: int, S_kv: int, D: int, type_siz
     for br, bc, nw, st, pipe, mfma, qs in _enumerate(FA_DOMAINS, cons, count, backend):
         cfg = FAConfig(Br=br, Bc=bc, num_warps=nw, stages=st, pipe=int(pipe), mfma=mfma,
                        q_in_smem=bool(qs))
-        results.append(cfg)
+        forms = [cfg]
         # the plain ring loop in its one-copy form, where the unrolled one is expected to
         # run out of registers (it interacts with no other constraint: expanded here)
         if int(pipe) == 0 and st >= 2 and register_fill(cfg, D) >= 0.95:
-            results.append(replace(cfg, roll=True))
+            forms.append(replace(cfg, roll=True))
         # the next tile's loads dealt over the first matrix-instruction groups of a step
         if default_spread(cfg):
-            results.append(replace(cfg, spread=default_spread(cfg)))
+            forms.append(replace(cfg, spread=default_spread(cfg)))
+        # the plain ring loops with the tile's exponentials taken against the running max as
+        # it stands (no max of the tile first; a tile that outgrew it is done again)
+        if int(pipe) == 0 and st >= 2:
+            forms += [replace(f, trust=True) for f in forms]
+        results += forms
     return results

@@ -375,6 +375,11 @@ def fa_score(cfg, arch, shape, causal: bool = False) -> float:
     # plain loop with short (64-key, D = 64) steps, nothing or a little less elsewhere
     if getattr(cfg, "spread", 0):
         pipe *= 1.01 if int(cfg.pipe) == 2 else (1.02 if cfg.Bc * D <= 64 * 64 else 0.995)
+    # no max of the tile ahead of its exponentials (plain ring loops): +3.6 % on the full
+    # S = 4096 shapes at both head dims; under the causal mask nothing is gained and the
+    # second pass the step keeps in reserve costs 4-7 %
+    if getattr(cfg, "trust", False):
+        pipe *= 1.035 if not causal else 0.95
     if not getattr(cfg, "swizzle", True):
         pipe *= 0.5  # linear LDS rows: every fragment read is a multi-way bank conflict
     sync = 1.0 / (1.0 + getattr(arch, "fa_cta_sync_penalty", 0.0) * cfg.num_warps / 4 / wgs)

@@ -17,6 +17,9 @@
 //   DECA_SPREAD         n > 0: the K/V loads of the next tile are dealt over the first n
 //                       matrix-instruction groups of a step instead of issued in one burst
 //                       behind the barrier (plain ring loops and slot loop)
+//   DECA_TRUST          1 (plain ring loops): a tile's exponentials are taken against the
+//                       running max as it stands, without looking at the tile's own max
+//                       first; a tile that turns out to have outgrown it is done again
 //   DECA_CAUSAL         1: key j visible to query i iff j <= i (SQ == SKV)
 //   DECA_SCALE          softmax scale
 //   DECA_PIPE           1: S^T of the next tile is computed before the softmax of
@@ -86,6 +89,9 @@
 #ifndef DECA_SPREAD
 #define DECA_SPREAD 0
 #endif
+#ifndef DECA_TRUST
+#define DECA_TRUST 0
+#endif
 #ifndef DECA_MIN_WAVES
 #define DECA_MIN_WAVES 1  // waves per SIMD the register allocation must leave room for
 #endif
@@ -140,6 +146,7 @@ static_assert(DECA_SQ % BR == 0 && DECA_SKV % BC == 0, "tiles must divide the se
 static_assert(TILE_CHUNKS % NT == 0, "loader coverage");
 static_assert(STAGES >= 1 && STAGES <= 3, "K/V ring depth");
 static_assert(STAGES < 3 || DECA_PIPE == 0, "three stages: plain loop only");
+static_assert(!DECA_TRUST || (DECA_PIPE == 0 && STAGES >= 2), "trust: a form of the plain ring loops");
 static_assert(STAGES < 3 || 4 * KV_IT <= 63, "two tile pairs in flight fit the 6-bit counter");
 static_assert(!DECA_CAUSAL || DECA_SQ == DECA_SKV, "causal needs S_q == S_kv");
 static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
@@ -440,7 +447,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
   // K: row = kt*32 + lane%32, chunk = (ks*2 + half) ^ k_swz(row); the row bits used by
   // the swizzle do not depend on kt (k_swz has period 16).
   // (16x16x32: row = kt*16 + lane%16, chunk = (ks*4 + lane/16) ^ k_swz(row))
-  const unsigned k_lane_base = static_cast<unsigned>(lq * CPR + (lg ^ k_swz(lq))) * 16u;
+  unsigned k_lane_base = static_cast<unsigned>(lq * CPR + (lg ^ k_swz(lq))) * 16u;
   auto k_frag_offset = [&](int ks, int kt) __attribute__((always_inline)) {
     return (k_lane_base ^ k_xor_const(ks * K_CHUNKS_PER_STEP)) + k_add_const(ks * K_CHUNKS_PER_STEP) +
            static_cast<unsigned>(kt * TQ * CPR * 16);
@@ -599,6 +606,87 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
           for (int e = 0; e < ACC_N; ++e) o_acc[dt][mq][e] *= alpha[mq];
     }
   };
+#if DECA_TRUST
+  // The softmax of a tile taken on trust (`with_max` false): exponentials against the
+  // running max as it stands, no max of the tile at all.  A lane's p are then bounded by
+  // their own sum, which is looked at afterwards: while no lane of the wave has more than
+  // 2^15 in it, every p fits fp16 and the running max may stay (alpha = 1, nothing to
+  // rescale); otherwise the call returns true with l and O untouched, and the caller
+  // computes S^T again and comes back with `with_max` true, which is `softmax` above.
+  // O / l is the same quotient either way.
+  auto softmax_flex = [&](acc_t (&s_acc)[KT][MQ], half8 (&pf)[KK][MQ], bool with_max) __attribute__((always_inline)) -> bool {
+    float alpha[MQ], tile_sum[MQ];
+#pragma unroll
+    for (int mq = 0; mq < MQ; ++mq) alpha[mq] = 1.0f;
+    if (with_max) {
+#pragma unroll
+      for (int mq = 0; mq < MQ; ++mq) {
+        float mx = s_acc[0][mq][0];
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+          for (int e = 0; e < ACC_N; ++e) mx = fmaxf(mx, s_acc[kt][mq][e]);
+        mx = max_over_query(mx);
+        const float m_new = lazy_max(m_i[mq], mx);
+        alpha[mq] = __builtin_amdgcn_exp2f((m_i[mq] - m_new) * SL2);
+        m_i[mq] = m_new;
+      }
+    }
+    bool over = false;
+#pragma unroll
+    for (int mq = 0; mq < MQ; ++mq) {
+      const float msl = m_i[mq] * SL2;
+      float sum = 0.0f;
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt) {
+#pragma unroll
+        for (int e = 0; e < ACC_N; ++e) {
+          const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s_acc[kt][mq][e], SL2, -msl));
+          s_acc[kt][mq][e] = p;
+          sum += p;
+        }
+#if !DECA_MFMA16
+#pragma unroll
+        for (int hh = 0; hh < 2; ++hh) {
+          half8 h;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) h[e] = static_cast<_Float16>(s_acc[kt][mq][hh * 8 + e]);
+          pf[kt * 2 + hh][mq] = h;
+        }
+#endif
+      }
+#if DECA_MFMA16
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk) {
+        half8 h;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          h[e] = static_cast<_Float16>(s_acc[2 * kk][mq][e]);
+          h[4 + e] = static_cast<_Float16>(s_acc[2 * kk + 1][mq][e]);
+        }
+        pf[kk][mq] = h;
+      }
+#endif
+      tile_sum[mq] = sum;
+      over |= !(sum <= 32768.0f);  // also true for inf and NaN
+    }
+    if (!with_max && __builtin_amdgcn_ballot_w64(over) != 0) return true;
+#pragma unroll
+    for (int mq = 0; mq < MQ; ++mq) l_i[mq] = l_i[mq] * alpha[mq] + tile_sum[mq];
+    bool moved = false;
+#pragma unroll
+    for (int mq = 0; mq < MQ; ++mq) moved |= (alpha[mq] != 1.0f);
+    if (__builtin_amdgcn_ballot_w64(moved) != 0) {
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int mq = 0; mq < MQ; ++mq)
+#pragma unroll
+          for (int e = 0; e < ACC_N; ++e) o_acc[dt][mq][e] *= alpha[mq];
+    }
+    return false;
+  };
+#endif
   // O^T += V^T P^T for the tile in V slot `vslot`.  k-slot (half, e) of step kk
   // is key row kk*16 + (e/4)*8 + half*4 + e%4: the order in which the S^T
   // accumulator registers hold the keys.
@@ -676,6 +764,34 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
     if (skip) return;
     acc_t s_acc[KT][MQ];
     half8 pf[KK][MQ];
+#if DECA_TRUST
+    // The first tile has no running max to trust and takes its own.  Every other tile is
+    // taken on trust first; one that outgrew the running max goes round again: S^T is
+    // computed once more (p overwrote it; its K tile is still in the slot), then its max.
+    bool in_full = j == 0;
+#if DECA_CAUSAL
+    // a tile that reaches the diagonal for this wave needs the mask: never on trust
+    in_full |= (j + 1) * BC - 1 > qt * BR + wave_u * WQ;
+#endif
+    bool request = more;  // the next tile's loads ride on the first pass only
+#pragma unroll 1
+    for (;;) {
+      // (an opaque copy per pass: the fragment addresses derived from it are then no loop
+      // invariants, which the optimiser would compute ahead of the loop and keep in registers)
+      asm volatile("" : "+v"(k_lane_base));
+#if DECA_SPREAD > 0
+      compute_s(s_acc, slot, [&](int i) __attribute__((always_inline)) {
+        if (i < SPREAD_N && request) issue_kv_share(ahead, fill, ahead, fill, i, SPREAD_N);
+      });
+#else
+      compute_s(s_acc, slot, nothing);
+#endif
+      if (in_full) mask_s(s_acc, j);
+      if (!softmax_flex(s_acc, pf, in_full)) break;
+      in_full = true;
+      request = false;
+    }
+#else
 #if DECA_SPREAD > 0
     // the requested tile's loads ride on the first SPREAD_N groups of S^T instructions
     compute_s(s_acc, slot, [&](int i) __attribute__((always_inline)) {
@@ -686,6 +802,7 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
 #endif
     mask_s(s_acc, j);
     softmax(s_acc, pf);
+#endif
     compute_pv(pf, slot);
   };
 #endif

@@ -101,7 +101,8 @@ def parse_config(operator: str, text: str):
                       num_warps=int(pairs.pop("warps")), stages=int(pairs.pop("stages")),
                       q_in_smem=bool(int(pairs.pop("q_smem", 0))), swizzle=bool(int(pairs.pop("swz", 1))),
                       pipe=int(pairs.pop("pipe", 0)), mfma=int(pairs.pop("mfma", 32)),
-                      roll=bool(int(pairs.pop("roll", 0))), spread=int(pairs.pop("spread", 0)))
+                      roll=bool(int(pairs.pop("roll", 0))), spread=int(pairs.pop("spread", 0)),
+                      trust=bool(int(pairs.pop("trust", 0))))
     if pairs:
         raise ValueError(f"unknown fields in {operator} config {text!r}: {sorted(pairs)}")
     cfg = cls(**fields)

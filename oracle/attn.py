@@ -63,7 +63,8 @@ def attention_f32(q, k, v, scale=None, causal=False) -> np.ndarray:
 
 
 def flash_blockwise(q, k, v, scale=None, causal=False, Br=128, Bc=64, lazy_tau=0.0,
-                    max_every=1) -> np.ndarray:
+                    max_every=1, trust_bound=None, wave_rows=32, key_groups=(8, 4),
+                    stats=None) -> np.ndarray:
     """The tiled online-softmax recurrence; returns fp32 values rounded to fp16.
 
     `lazy_tau` = 0 is the reference's update m' = max(m, rowmax S)
@@ -73,7 +74,16 @@ def flash_blockwise(q, k, v, scale=None, causal=False, Br=128, Bc=64, lazy_tau=0
     the same quotient with p <= 2^lazy_tau.  `max_every` > 1 looks at a tile's
     max only in every `max_every`-th tile (a variant that was considered for the
     kernel and is NOT safe: nothing bounds p in the tiles between, see
-    tests/test_oracle_attn.py)."""
+    tests/test_oracle_attn.py).
+
+    `trust_bound` (the kernel's `FAConfig.trust`, bound 2^15): every tile but the first (and,
+    under the causal mask, but those that reach the diagonal for a wave) has its exponentials
+    taken against the running max as it stands, without its own max.  The p of a lane are
+    bounded by their sum, so a wave (`wave_rows` query rows) accepts the tile while no lane's
+    sum exceeds the bound -- a lane holds the keys k of the tile with
+    (k % key_groups[0]) // key_groups[1] == its group: (8, 4) for 32x32x16 tiles, (16, 4) for
+    16x16x32 -- and otherwise does the tile again with its max (lazy rule).  `stats`, a dict,
+    receives the number of (wave, tile) pairs taken on trust and of those done again."""
     q = np.asarray(q, np.float32)
     k = np.asarray(k, np.float32)
     v = np.asarray(v, np.float32)
@@ -101,6 +111,24 @@ def flash_blockwise(q, k, v, scale=None, causal=False, Br=128, Bc=64, lazy_tau=0
                         m_new = m
                     elif lazy_tau > 0:
                         m_new = np.where((m_new - m) * sl2 > np.float32(lazy_tau), m_new, m)
+                    if trust_bound is not None and tile > 0:
+                        # per wave: trust the running max unless the tile needs the mask or a
+                        # lane's sum of p = exp2((s - m) sl2) says that some p may not fit fp16
+                        group = (np.arange(s.shape[1]) % key_groups[0]) // key_groups[1]
+                        with np.errstate(over="ignore"):
+                            p_old = np.exp2(s * sl2 - (m * sl2)[:, None], dtype=np.float32)
+                        for w0 in range(0, s.shape[0], wave_rows):
+                            w = slice(w0, w0 + wave_rows)
+                            if causal and k0 + s.shape[1] - 1 > q0 + w0:
+                                continue
+                            sums = np.stack([p_old[w][:, group == g].sum(axis=-1, dtype=np.float32)
+                                             for g in range(group.max() + 1)])
+                            if stats is not None:
+                                stats["trusted"] = stats.get("trusted", 0) + 1
+                            if np.all(sums <= np.float32(trust_bound)):
+                                m_new[w] = m[w]
+                            elif stats is not None:
+                                stats["redone"] = stats.get("redone", 0) + 1
                     alpha = np.exp2((m - m_new) * sl2, dtype=np.float32)
                     p = np.exp2(s * sl2 - (m_new * sl2)[:, None], dtype=np.float32)
                     l = l * alpha + p.sum(axis=-1, dtype=np.float32)

@@ -262,6 +262,22 @@ FA_CASES = [
     (2, 2, 512, 512, 64, False, FAConfig(256, 64, 4, 3, spread=4)),
     (1, 2, 512, 512, 128, True, FAConfig(128, 64, 4, 3, mfma=16, spread=2)),
     (1, 2, 256, 320, 64, False, FAConfig(128, 64, 2, 3, spread=100)),
+    # exponentials against the running max as it stands (`trust`): both tile forms, two and
+    # three stages, unrolled and rolled, with the load window and the staged Q tile, full and
+    # causal (tiles that reach the diagonal always take their max), D = 64 / 128 / 192,
+    # one, two and an odd number of tiles
+    (1, 2, 512, 512, 128, False, FAConfig(256, 128, 8, 2, mfma=16, roll=True, trust=True)),
+    (2, 2, 512, 512, 64, False, FAConfig(256, 64, 4, 3, trust=True)),
+    (1, 2, 512, 512, 128, True, FAConfig(256, 128, 8, 2, mfma=16, roll=True, trust=True)),
+    (2, 2, 512, 512, 64, True, FAConfig(256, 64, 4, 3, trust=True)),
+    (1, 2, 256, 320, 64, False, FAConfig(128, 64, 4, 2, trust=True)),
+    (1, 2, 256, 320, 128, False, FAConfig(128, 64, 4, 2, mfma=16, spread=4, trust=True)),
+    (1, 2, 512, 512, 128, True, FAConfig(256, 64, 8, 2, spread=4, trust=True)),
+    (1, 2, 256, 256, 192, False, FAConfig(128, 32, 4, 2, q_in_smem=True, mfma=16, trust=True)),
+    (1, 2, 256, 256, 192, True, FAConfig(128, 32, 4, 3, q_in_smem=True, trust=True)),
+    (1, 2, 128, 64, 64, False, FAConfig(64, 64, 2, 3, trust=True)),
+    (1, 2, 128, 128, 128, True, FAConfig(64, 64, 2, 2, mfma=16, roll=True, trust=True)),
+    (1, 3, 128, 640, 128, False, FAConfig(64, 64, 2, 3, roll=True, trust=True)),
     # linear LDS rows (no swizzle): both row lengths, both tile forms, with and without the
     # staged Q tile
     (1, 2, 256, 256, 128, True, FAConfig(128, 64, 4, 2, swizzle=False)),
@@ -283,6 +299,9 @@ FA_FULL = [
     (4, 16, 4096, 4096, 64, True, FAConfig(256, 64, 4, 3, q_in_smem=True)),
     (4, 16, 4096, 4096, 128, True, FAConfig(256, 64, 8, 2, pipe=2, spread=8)),
     (4, 16, 4096, 4096, 64, False, FAConfig(256, 64, 4, 2, spread=4)),
+    (4, 16, 4096, 4096, 128, False, FAConfig(256, 128, 8, 2, mfma=16, roll=True, trust=True)),
+    (4, 16, 4096, 4096, 64, False, FAConfig(256, 64, 4, 3, trust=True)),
+    (4, 16, 4096, 4096, 64, True, FAConfig(256, 64, 4, 2, spread=4, trust=True)),
 ]
 
 

@@ -122,6 +122,41 @@ def test_flash_attn_growing_max(pipe, causal):
     assert np.abs(got - ref).max() <= GATE
 
 
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("mfma", [32, 16])
+def test_flash_attn_trusted_max_is_outgrown(mfma, causal):
+    """`trust`: keys that grow along the sequence outgrow the running max again and again, so
+    tiles taken on trust fail their check (a lane's sum of p beyond 2^15) and are done again
+    with their max; and scores far from zero (|s| ~ 60) make the very first trusted tile fail.
+    Both must come out within the gate, as with the max taken ahead of every tile."""
+    from deca_amd.kernels.attn_bench import make_qkv_cpu
+
+    B, H, S, _, D, _, cfg = next(c for c in FA_CASES
+                                 if c[6].trust and c[6].mfma == mfma and c[5] == causal and c[2] == c[3] >= 512)
+    print(f"case fa trusted max outgrown S{S} D{D} causal={causal} {cfg}", flush=True)
+    q, k, v = make_qkv_cpu(B, H, S, S, D, seed=21)
+    ramp = torch.linspace(0.2, 6.0, S)[None, None, :, None]
+    kr = (k.float() * ramp).half()
+    # the check does fire on this input: the CPU restatement of the same rule counts the tiles
+    st = {}
+    want = oa.flash_blockwise(_f32(q), _f32(kr), _f32(v), None, causal, Br=cfg.Br, Bc=cfg.Bc, lazy_tau=8.0,
+                              trust_bound=2.0 ** 15, wave_rows=cfg.Br // cfg.num_warps,
+                              key_groups=(16, 4) if mfma == 16 else (8, 4), stats=st)
+    assert st["redone"] > 0
+    ref = oa.attention_f32(_f32(q), _f32(kr), _f32(v), None, causal)
+    got = _f32(_run(B, H, S, S, D, causal, cfg, q, kr, v))
+    assert np.isfinite(got).all()
+    # (peaked rows: |o| reaches 3 and more, where the fp16 grid is 2e-3 and wider -- the gate is
+    # relative there, as in test_flash_attn_large_scores)
+    assert (np.abs(got - ref) <= GATE * np.maximum(1.0, np.abs(ref))).all()
+    assert (np.abs(got - want) <= GATE * np.maximum(1.0, np.abs(want))).all()
+    q6, k6 = (q.float() * 6).half(), (k.float() * 6).half()
+    got = _f32(_run(B, H, S, S, D, causal, cfg, q6, k6, v))
+    ref = oa.attention_f32(_f32(q6), _f32(k6), _f32(v), None, causal)
+    assert np.isfinite(got).all()
+    assert (np.abs(got - ref) <= GATE * np.maximum(1.0, np.abs(ref))).all()
+
+
 @pytest.mark.parametrize("B,H,Sq,Skv,D,causal,cfg", FA_FULL, ids=lambda v: str(v))
 def test_flash_attn_full_size(B, H, Sq, Skv, D, causal, cfg):
     """Benchmark shapes: a few (batch, head) slices against the CPU checker,

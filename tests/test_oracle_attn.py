@@ -74,6 +74,42 @@ def test_running_max_must_see_every_tile():
     assert (s.reshape(64, 16, 32).max(-1)[:, 1:] - seen[:, :-1]).max() > 16 + 8
 
 
+@pytest.mark.parametrize("groups", [(8, 4), (16, 4)])
+def test_trusted_running_max_is_checked_after_the_fact(groups):
+    """`FAConfig.trust`: a tile's exponentials against the running max as it stands, without
+    the tile's own max.  What makes that safe is the check behind it -- a lane's p are bounded
+    by their sum, and a wave whose lane sums pass 2^15 does the tile again with its max.  On
+    ordinary inputs no tile is done again and the result is the eager recurrence's; on keys
+    that grow along the sequence tiles are done again and the result stays within the gate;
+    with the check taken away (an infinite bound) the same input pushes p past the fp16
+    range and the output is lost."""
+    q, k, v = _qkv(1, 2, 128, 512, 64, seed=2)
+    for causal in (False, True):
+        kk, vv = (k[:, :, :128], v[:, :, :128]) if causal else (k, v)
+        ref = oa.attention_f32(q, kk, vv, None, causal)
+        st = {}
+        got = oa.flash_blockwise(q, kk, vv, None, causal, Br=64, Bc=32, lazy_tau=8.0, trust_bound=2.0 ** 15,
+                                 key_groups=groups, stats=st)
+        assert np.abs(got - ref).max() < 2e-3
+        assert st["trusted"] > 0 and st.get("redone", 0) == 0
+    # growing keys: the running max is outgrown again and again
+    q, k, v = _qkv(1, 1, 64, 512, 64, seed=4)
+    k = k * np.linspace(0.2, 14.0, 512, dtype=np.float32)[None, None, :, None]
+    k = k.astype(np.float16).astype(np.float32)
+    ref = oa.attention_f32(q, k, v, None, False)
+    st = {}
+    with np.errstate(over="ignore", invalid="ignore"):
+        checked = oa.flash_blockwise(q, k, v, None, False, Br=64, Bc=32, lazy_tau=8.0, trust_bound=2.0 ** 15,
+                                     key_groups=groups, stats=st)
+        blind = oa.flash_blockwise(q, k, v, None, False, Br=64, Bc=32, lazy_tau=8.0, trust_bound=np.inf,
+                                   key_groups=groups)
+    assert np.abs(checked - ref).max() < 2e-3
+    assert 0 < st["redone"] < st["trusted"]
+    assert not np.isfinite(blind).all() or np.abs(blind - ref).max() > 2e-3
+    # the bound: while every lane sum stays within 2^15, every p does, and fp16 holds it
+    assert np.float16(2.0 ** 15) == 2.0 ** 15 and np.isfinite(np.float16(2.0 ** 15))
+
+
 @pytest.mark.parametrize("causal", [False, True])
 def test_lazy_running_max_is_the_same_quotient(causal):
     """The kernel's lazy running max against the reference's eager one: keys grow

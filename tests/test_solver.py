@@ -153,14 +153,19 @@ def test_flash_attn_configs_are_valid(D, S):
         regs = (fa.est_regs_per_thread(cfg, D) + 7) // 8 * 8
         if regs * -(-nw // 4) > 512 or not fa.expect_spill_free(cfg, D):
             continue
-        want.add(cfg)
+        forms = [cfg]
         # the one-copy form of the plain ring loop, where the unrolled one is tight
         if pipe == 0 and st >= 2 and fa.register_fill(cfg, D) >= 0.95:
-            want.add(replace(cfg, roll=True))
+            forms.append(replace(cfg, roll=True))
         # the load window of the two-stage plain and slot loops
         if st == 2 and pipe in (0, 2):
-            want.add(replace(cfg, spread=8 if pipe == 2 else 4))
+            forms.append(replace(cfg, spread=8 if pipe == 2 else 4))
+        # every plain ring loop also without the tile's max ahead of its exponentials
+        if pipe == 0 and st >= 2:
+            forms += [replace(f, trust=True) for f in forms]
+        want.update(forms)
     assert set(configs) == want
+    assert all(int(c.pipe) == 0 and c.stages >= 2 for c in configs if c.trust)
     # the reference's knobs are all in the search (Solver.py:330-336), except linear LDS rows
     assert {c.stages for c in configs} == {1, 2, 3}
     assert {c.q_in_smem for c in configs} == {False, True} and all(c.swizzle for c in configs)
@@ -285,6 +290,17 @@ def test_flash_attn_knobs_of_the_reference():
     assert dict(fa.make_flash_attn_fwd(4, 16, 4096, 4096, 128, sp).defines)["DECA_SPREAD"] == 8
     assert str(sp).endswith(",pipe=2,spread=8")
     for bad in (replace(base, pipe=1, spread=4), replace(base, stages=1, spread=4)):
+        with pytest.raises(AssertionError):
+            fa.check_config(bad, 4096, 4096, 128)
+    # no max ahead of a tile's exponentials: plain ring loops only (the slot loop consumes
+    # P while the check is still out, the one-stage loop has no ring step to repeat in)
+    tr = replace(base, mfma=16, roll=True, trust=True)
+    assert dict(fa.make_flash_attn_fwd(4, 16, 4096, 4096, 128, tr).defines)["DECA_TRUST"] == 1
+    assert "DECA_TRUST" not in dict(fa.make_flash_attn_fwd(4, 16, 4096, 4096, 128, base).defines)
+    assert str(tr).endswith(",mfma=16,roll=1,trust=1")
+    fa.check_config(replace(deep, trust=True), 4096, 4096, 128)
+    for bad in (replace(base, pipe=2, trust=True), replace(base, pipe=1, trust=True),
+                replace(base, stages=1, trust=True)):
         with pytest.raises(AssertionError):
             fa.check_config(bad, 4096, 4096, 128)
     # three stages belong to the plain loop; four do not exist

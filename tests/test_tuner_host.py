@@ -339,6 +339,8 @@ def test_config_strings_parse_back():
         ("flash_attn", FAConfig(256, 64, 8, 2, pipe=2)),
         ("flash_attn", FAConfig(128, 128, 4, 1)),
         ("flash_attn", FAConfig(256, 128, 8, 2, mfma=16, roll=True)),
+        ("flash_attn", FAConfig(256, 64, 4, 3, trust=True)),
+        ("flash_attn", FAConfig(256, 64, 4, 2, spread=4, trust=True)),
     ]
     for op, cfg in cases:
         assert tuned.parse_config(op, str(cfg)) == cfg
