@@ -80,10 +80,16 @@ def pair_effects(run: dict, old: str, new: str) -> dict:
     """What one field of the configuration does, everything else equal: over all measured
     pairs of configurations whose text differs only in `old` -> `new` (e.g. "stages=2",
     "stages=3"), the ratios new / old, the pair with the fastest `new` member, and the
-    same ratios among pairs whose better member is within 10 % of the run's best."""
+    same ratios among pairs whose better member is within 10 % of the run's best.  An empty
+    `old` pairs the configurations that carry `new` with their twins without it (fields that
+    are only printed when set, e.g. "" -> "trust=1")."""
     thr = dict(run["measured"])
     best = max(thr.values())
-    pairs = [(c, c.replace(old, new)) for c in thr if old in c.split(",") and c.replace(old, new) in thr]
+    if old:
+        pairs = [(c, c.replace(old, new)) for c in thr if old in c.split(",") and c.replace(old, new) in thr]
+    else:
+        pairs = [(",".join(f for f in c.split(",") if f != new), c) for c in thr if new in c.split(",")]
+        pairs = [(a, b) for a, b in pairs if a in thr]
     ratios = sorted(thr[b] / thr[a] for a, b in pairs)
     near = sorted(thr[b] / thr[a] for a, b in pairs if max(thr[a], thr[b]) >= 0.9 * best)
     top = max(pairs, key=lambda ab: thr[ab[1]], default=None)

@@ -169,3 +169,19 @@ def test_rank_report_reads_the_drivers_output():
     assert rr.quality(runs[1])["best_rank"] == 1
     lines = rr.table(runs).splitlines()
     assert len(lines) == 4 and "| 244 | 4 | 2 |" in lines[2]
+
+
+def test_rank_report_pairs_configurations_that_differ_in_one_field():
+    """`pair_effects`: ratios over twins that differ in one field, also for a field that is
+    only printed when it is set (an empty old value)."""
+    from deca_amd.cost_model import rank_report as rr
+
+    run = {"what": "x", "solutions": 6, "unit": "TFLOPS", "measured": [
+        ("Br=256,stages=2", 1000.0), ("Br=256,stages=3", 900.0), ("Br=256,stages=2,trust=1", 1040.0),
+        ("Br=128,stages=2", 500.0), ("Br=128,stages=2,trust=1", 490.0), ("Br=64,stages=3,trust=1", 100.0)]}
+    e = rr.pair_effects(run, "stages=2", "stages=3")
+    assert e["pairs"] == 1 and abs(e["median"] - 0.9) < 1e-12
+    e = rr.pair_effects(run, "", "trust=1")
+    assert e["pairs"] == 2 and abs(e["min"] - 0.98) < 1e-12 and abs(e["max"] - 1.04) < 1e-12
+    assert e["near_pairs"] == 1 and e["top"] == ("Br=256,stages=2,trust=1", 1040.0, 1000.0)
+    assert " -> trust=1 | 2 |" in rr.pairs_table([run], [":trust=1"])
