@@ -154,8 +154,8 @@ def run_rowwise(wl, steps, warmup, with_cpu):
     for i in range(nsets):
         inputs = make_inputs(op, M, N, dtype, seed=i, std=2.0 if op == "softmax" else 1.0)
         sets.append((*inputs, torch.empty_like(inputs[0])))
-    # wall time per step, and kernel time from HIP events around the same launches
-    wall, t_rot = _timed_steps(kern, sets, steps, warmup)
+    # wall time per step, and kernel time from events around the same launches
+    wall, t_rot, first = _timed_steps(kern, sets, steps, warmup)
     t_same = kern.time(sets[:1], steps)
     gbs = nbytes / wall / 1e9
     res = {
@@ -170,7 +170,7 @@ def run_rowwise(wl, steps, warmup, with_cpu):
             "bound": "hbm", "achieved": nbytes / t_rot / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": nbytes / t_rot / 1e9 / HBM_PEAK_GBS, "traffic": None,
             "kernel_us": t_rot * 1e6, "kernel_us_same_buffers": t_same * 1e6,
-            "algorithmic_bytes": nbytes, "buffer_sets": nsets,
+            "algorithmic_bytes": nbytes, "buffer_sets": nsets, "timed_launches": [first, steps],
         },
     }
     res["roofline"].update(_board(kern, sets))
@@ -182,8 +182,12 @@ def run_rowwise(wl, steps, warmup, with_cpu):
 
 
 def _timed_steps(kern, sets, steps, warmup):
-    """(wall seconds per step, event seconds per launch) over `steps` launches
-    cycling through the argument sets."""
+    """(wall seconds per step, event seconds per launch, index of the first timed launch
+    among the kernel object's launches) over the same `steps` back-to-back launches cycling
+    through the argument sets: the host clock is read, with the device idle, on either side
+    of the region, and two events are recorded on the launch stream (torch's current stream)
+    directly before the first and after the last launch inside it (`deca_launch_between`), so
+    the event time can never exceed the wall time."""
     import torch
 
     n = len(sets)
@@ -199,13 +203,18 @@ def _timed_steps(kern, sets, steps, warmup):
         torch.cuda.synchronize()
     for i in range(warmup):
         kern(*sets[i % n])
+    packed = kern.pack(sets)
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()  # (an event is created at its first record: not inside the timed region)
+    stop.record()
+    run = kern.batch_call(packed, steps, start, stop)
     torch.cuda.synchronize()
+    first = kern.launches
     t0 = time.perf_counter()
-    for i in range(steps):
-        kern(*sets[i % n])
+    run()
     torch.cuda.synchronize()
     wall = (time.perf_counter() - t0) / steps
-    return wall, kern.time(sets, steps)
+    return wall, start.elapsed_time(stop) * 1e-3 / steps, first
 
 
 def run_gemm(wl, steps, warmup, with_cpu):
@@ -220,7 +229,7 @@ def run_gemm(wl, steps, warmup, with_cpu):
     short = "bf16" if wl["dtype"] == "bfloat16" else "f16"
     a, b = make_inputs(M, N, K, seed=0, dist="uniform", dtype=tdt)
     c = torch.empty(M, N, dtype=tdt, device="cuda")
-    wall, t_k = _timed_steps(kern, [(a, b, c)], steps, warmup)
+    wall, t_k, first = _timed_steps(kern, [(a, b, c)], steps, warmup)
     flops = gemm_flops(M, N, K)
     board = _board(kern, [(a, b, c)])
     # the same kernel on the reference's operand distribution, N(0,1) (gemm_bench.py:26-31):
@@ -236,6 +245,7 @@ def run_gemm(wl, steps, warmup, with_cpu):
         "roofline": {"bound": "mfma", "achieved": flops / t_k / 1e12, "peak": MFMA_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": flops / t_k / 1e12 / MFMA_PEAK_TFLOPS,
                      "traffic": None, "kernel_us": t_k * 1e6, "algorithmic_flops": flops,
+                     "timed_launches": [first, steps],
                      "achieved_normal_inputs": flops / t_n01 / 1e12},
     }
     res["roofline"].update(board)
@@ -256,7 +266,7 @@ def run_fa(wl, steps, warmup, with_cpu):
     kern = build_flash_attn(_spec(wl))
     q, k, v = make_qkv(B, H, S, S, D, seed=0)
     o = torch.empty_like(q)
-    wall, t_k = _timed_steps(kern, [(q, k, v, o)], steps, warmup)
+    wall, t_k, first = _timed_steps(kern, [(q, k, v, o)], steps, warmup)
     flops = attn_flops(B, H, S, S, D, causal)
     res = {
         "workload": wl["name"],
@@ -265,7 +275,8 @@ def run_fa(wl, steps, warmup, with_cpu):
         "dtype": "f16 in/out, f32 accumulate", "config": str(wl["cfg"]),
         "roofline": {"bound": "mfma", "achieved": flops / t_k / 1e12, "peak": MFMA_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": flops / t_k / 1e12 / MFMA_PEAK_TFLOPS,
-                     "traffic": None, "kernel_us": t_k * 1e6, "algorithmic_flops": flops},
+                     "traffic": None, "kernel_us": t_k * 1e6, "algorithmic_flops": flops,
+                     "timed_launches": [first, steps]},
     }
     res["roofline"].update(_board(kern, [(q, k, v, o)]))
     if with_cpu:

@@ -119,14 +119,17 @@ def bench_record(log_path: str):
     return rec
 
 
-def event_timed_durations(trace_rows: list, steps: int, rowwise: bool) -> list:
-    """Durations (ns) of the launches bench.py timed with HIP events: the last `steps`
-    launches of the run, or -- row-wise workloads, which are timed once more over a
-    single buffer set afterwards -- the `steps` before those."""
+def event_timed_durations(trace_rows: list, first: int, count: int) -> list:
+    """Durations (ns) of the launches bench.py timed: `count` launches of the kernel under
+    test from its `first` one on (the record's `roofline.timed_launches`; spin-up and warm-up
+    launches come before them, the row-wise pass over a single buffer set and the GEMM's
+    pass on N(0,1) operands after)."""
     mine = sorted((r for r in trace_rows if r["Kernel_Name"].startswith("deca_main")),
                   key=lambda r: int(r["Start_Timestamp"]))
     durs = [int(r["End_Timestamp"]) - int(r["Start_Timestamp"]) for r in mine]
-    return durs[-2 * steps:-steps] if rowwise else durs[-steps:]
+    if not 0 <= first <= first + count <= len(durs):
+        raise ValueError(f"the trace holds {len(durs)} launches, the record times {first}..{first + count}")
+    return durs[first:first + count]
 
 
 def counter_means(counter_rows: list, kernel_prefix: str | None = None) -> dict:
@@ -189,7 +192,7 @@ def summary_text(workload: str, out_dir: str, kernel_config: str | None = None) 
     stats = _rows(os.path.join(out_dir, "trace", "out_kernel_stats.csv"))
     trace = _rows(os.path.join(out_dir, "trace", "out_kernel_trace.csv"))
     steps = int(rec["steps"])
-    ev = event_timed_durations(trace, steps, rowwise)
+    ev = event_timed_durations(trace, *rec["roofline"]["timed_launches"])
     fetch = counter_means(_rows(os.path.join(out_dir, "fetch", "out_counter_collection.csv")))
     write = counter_means(_rows(os.path.join(out_dir, "write", "out_counter_collection.csv")))
 
@@ -211,12 +214,14 @@ def summary_text(workload: str, out_dir: str, kernel_config: str | None = None) 
                  f"{r['MaxNs']} | {float(r['Percentage']):.2f} |")
     t += ["", "`deca_main` is the kernel under test; the others are torch's input generators. The "
           "statistics cover every launch of the run: 0.3 s of untimed spin-up (clocks still ramping), "
-          f"the warm-up steps, {steps} wall-timed steps, then the {steps} launches timed with HIP events"
-          + (f" over rotating buffers and {steps} more over one buffer set" if rowwise else "") + ".", "",
-          f"From `out_kernel_trace.csv` of the same run, the {len(ev)} event-timed launches"
-          + (" over rotating buffers" if rowwise else "")
-          + f" alone: average {_mean(ev):.0f} ns (min {min(ev)}, max {max(ev)}); bench.py reports "
-          f"kernel_us = {rec['roofline']['kernel_us']:.2f} for them.", "",
+          f"the warm-up steps, the {steps} timed steps (host clock and events around the same launches"
+          + (", rotating buffers)" if rowwise else ")")
+          + (f", then {steps} more over one buffer set" if rowwise else "")
+          + (", then the passes on N(0,1) operands" if kern == "gemm" else "") + ".", "",
+          f"From `out_kernel_trace.csv` of the same run, the {len(ev)} timed launches alone: average "
+          f"{_mean(ev):.0f} ns (min {min(ev)}, max {max(ev)}); bench.py reports kernel_us = "
+          f"{rec['roofline']['kernel_us']:.2f} for them (event span / {len(ev)}: it includes the gaps "
+          "between consecutive launches).", "",
           "## bench.py line of the same run (HIP-event timing on the launch stream)", "", "```",
           json.dumps(rec), "```", "", "## L2 <-> fabric traffic per dispatch (KiB as reported)", "",
           "| kernel | FETCH_SIZE mean | WRITE_SIZE mean | dispatches |", "|---|---|---|---|"]

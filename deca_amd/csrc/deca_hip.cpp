@@ -167,6 +167,26 @@ int deca_launch_timed(void* fn, unsigned gx, unsigned gy, unsigned gz, unsigned 
   return rc(e);
 }
 
+int deca_launch_between(void* fn, unsigned gx, unsigned gy, unsigned gz, unsigned bx, unsigned by,
+                        unsigned bz, unsigned lds_bytes, void* stream, void* const* args,
+                        unsigned nargs, unsigned nsets, unsigned iters, void* start_event,
+                        void* stop_event) {
+  if (!fn || !args || nsets == 0 || iters == 0 || !geometry_ok(gx, gy, gz, bx, by, bz, nargs))
+    return rc(hipErrorInvalidValue);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  hipFunction_t f = static_cast<hipFunction_t>(fn);
+  void* params[kMaxArgs];
+  hipError_t e = hipSuccess;
+  if (start_event) e = hipEventRecord(static_cast<hipEvent_t>(start_event), s);
+  for (unsigned i = 0; e == hipSuccess && i < iters; ++i) {
+    void* const* set = args + static_cast<size_t>(i % nsets) * nargs;
+    for (unsigned a = 0; a < nargs; ++a) params[a] = const_cast<void**>(&set[a]);
+    e = hipModuleLaunchKernel(f, gx, gy, gz, bx, by, bz, lds_bytes, s, params, nullptr);
+  }
+  if (e == hipSuccess && stop_event) e = hipEventRecord(static_cast<hipEvent_t>(stop_event), s);
+  return rc(e);
+}
+
 int deca_synchronize(void* stream) {
   if (stream) return rc(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
   return rc(hipDeviceSynchronize());

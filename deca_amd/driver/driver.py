@@ -65,6 +65,11 @@ C_API = {
         [c_void_p] + [c_uint] * 7 + [c_void_p, POINTER(c_void_p), c_uint, c_uint, c_uint,
                                      POINTER(c_float)],
     ),
+    "deca_launch_between": (
+        c_int,
+        [c_void_p] + [c_uint] * 7 + [c_void_p, POINTER(c_void_p), c_uint, c_uint, c_uint,
+                                     c_void_p, c_void_p],
+    ),
     "deca_synchronize": (c_int, [c_void_p]),
     "deca_error_string": (c_char_p, [c_int]),
 }
@@ -157,12 +162,18 @@ class HipDriver:
             "deca_launch",
         )
 
+    @staticmethod
+    def pack_sets(ptr_sets):
+        """(array of all pointers, pointers per set, number of sets) of a list of equally
+        long pointer tuples, in the layout `deca_launch_timed` / `deca_launch_between` read."""
+        nsets, n = len(ptr_sets), len(ptr_sets[0])
+        flat = [p for s in ptr_sets for p in s]
+        return (c_void_p * (nsets * n))(*flat), n, nsets
+
     def launch_timed(self, fn, grid, block, lds_bytes, stream, ptr_sets, iters) -> float:
         """Seconds per launch, averaged over `iters` back-to-back launches that
         cycle through `ptr_sets` (a list of equally long pointer tuples)."""
-        nsets, n = len(ptr_sets), len(ptr_sets[0])
-        flat = [p for s in ptr_sets for p in s]
-        arr = (c_void_p * (nsets * n))(*flat)
+        arr, n, nsets = self.pack_sets(ptr_sets)
         ms = c_float(0.0)
         self.check(
             self.lib.deca_launch_timed(
@@ -171,6 +182,24 @@ class HipDriver:
             "deca_launch_timed",
         )
         return ms.value / 1e3 / iters
+
+    def batch_call(self, fn, grid, block, lds_bytes, stream, packed, iters,
+                   start_event: int = 0, stop_event: int = 0):
+        """A callable without arguments that enqueues `iters` back-to-back launches cycling
+        through `packed` (from `pack_sets`) and returns without waiting.  `start_event` /
+        `stop_event` are hipEvent_t handles of the caller (0: none), recorded on the stream
+        directly before the first and after the last launch.  Every argument is converted
+        here, so that the call itself is one foreign-function call."""
+        arr, n, nsets = packed
+        cargs = ([fn] + [c_uint(v) for v in (*grid, *block, lds_bytes)]
+                 + [c_void_p(stream), arr, c_uint(n), c_uint(nsets), c_uint(iters),
+                    c_void_p(start_event or None), c_void_p(stop_event or None)])
+        entry, check = self.lib.deca_launch_between, self.check
+
+        def call():
+            check(entry(*cargs), "deca_launch_between")
+
+        return call
 
     def synchronize(self, stream: int = 0):
         self.check(self.lib.deca_synchronize(c_void_p(stream)), "deca_synchronize")
@@ -201,6 +230,7 @@ class LoadedKernel:
     def __init__(self, spec, path: str, device: int = 0):
         self.spec = spec
         self.path = path
+        self.launches = 0  # launches issued through this object so far
         self.drv = get_driver()
         self.drv.init(device)
         self.mod = self.drv.module_load(path)
@@ -239,6 +269,7 @@ class LoadedKernel:
         return [t.data_ptr() for t in tensors]
 
     def __call__(self, *tensors):
+        self.launches += 1
         self.drv.launch(
             self.fn, self.spec.grid, self.spec.block, self.spec.lds_bytes, self._stream(),
             self._ptrs(tensors),
@@ -247,10 +278,37 @@ class LoadedKernel:
     def time(self, tensor_sets, iters: int) -> float:
         """Average seconds per launch over `iters` back-to-back launches cycling
         through `tensor_sets` (list of argument tuples)."""
+        self.launches += iters
         return self.drv.launch_timed(
             self.fn, self.spec.grid, self.spec.block, self.spec.lds_bytes, self._stream(),
             [self._ptrs(ts) for ts in tensor_sets], iters,
         )
+
+    def pack(self, tensor_sets):
+        """The argument sets in the form `batch` takes (built once, outside a timed region);
+        the tensors must stay alive while it is in use."""
+        return self.drv.pack_sets([self._ptrs(ts) for ts in tensor_sets])
+
+    def batch_call(self, packed, iters: int, start=None, stop=None):
+        """A callable without arguments that enqueues `iters` back-to-back launches cycling
+        through the packed argument sets on the stream that is current now, and does not
+        wait.  `start` / `stop`: torch.cuda.Event objects that have been recorded before (an
+        event is created at its first record), recorded again directly before the first and
+        after the last launch.  Prepared outside a timed region, called inside it."""
+        run = self.drv.batch_call(
+            self.fn, self.spec.grid, self.spec.block, self.spec.lds_bytes, self._stream(), packed, iters,
+            0 if start is None else int(start.cuda_event), 0 if stop is None else int(stop.cuda_event),
+        )
+
+        def call():
+            self.launches += iters
+            run()
+
+        return call
+
+    def batch(self, packed, iters: int, start=None, stop=None) -> None:
+        """`batch_call(...)()`."""
+        self.batch_call(packed, iters, start, stop)()
 
     def close(self):
         if getattr(self, "mod", None) is not None and self.mod:

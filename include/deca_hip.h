@@ -118,6 +118,19 @@ int deca_launch_timed(void* fn, unsigned gx, unsigned gy, unsigned gz,
                       void* stream, void* const* args, unsigned nargs,
                       unsigned nsets, unsigned iters, float* ms_total);
 
+/* Enqueues the same batch as deca_launch_timed between two events of the caller
+ * (hipEvent_t handles, e.g. torch.cuda.Event.cuda_event; either may be NULL) and
+ * returns without waiting: the events are recorded on `stream` directly before
+ * the first and directly after the last launch, so that a caller who reads its
+ * own clock around the call gets event and host time over the same launches.
+ * The events stay the caller's.  Replaces the start.record() ... end.record()
+ * pair around the launches in bench_cuda (src/kernels/attn_bench.py:58-66). */
+int deca_launch_between(void* fn, unsigned gx, unsigned gy, unsigned gz,
+                        unsigned bx, unsigned by, unsigned bz, unsigned lds_bytes,
+                        void* stream, void* const* args, unsigned nargs,
+                        unsigned nsets, unsigned iters, void* start_event,
+                        void* stop_event);
+
 /* Blocks until `stream` is idle (NULL: the whole device). */
 int deca_synchronize(void* stream);
 

@@ -96,3 +96,29 @@ def test_attention_workload(name):
     assert torch.isfinite(o).all()
     ref = math_attention(q, k, v, wl["causal"])
     assert (o.float() - ref).abs().max().item() <= 2e-3
+
+
+def test_wall_and_event_times_cover_the_same_launches():
+    """bench.py reads the host clock around the very launches that its two events bracket, so
+    a workload's `kernel_us` can never exceed its `ms_per_step`."""
+    from deca_amd.driver.driver import load_kernel
+    from deca_amd.kernels.build import cached_build
+
+    wl = WORKLOADS["softmax_fp16_16384x4096"]
+    spec = bench._spec(wl)
+    kern = load_kernel(spec, cached_build(spec))
+    x = torch.randn(wl["M"], wl["N"], device="cuda").to(torch.float16)
+    sets = [(x, torch.empty_like(x)) for _ in range(2)]
+    for steps in (1, 5, 20):
+        before = kern.launches
+        wall, t_k, first = bench._timed_steps(kern, sets, steps, 2)
+        assert 0 < t_k <= wall
+        assert wall < 50 * t_k  # and the host's share of a short region stays bounded
+        assert before < first and kern.launches == first + steps
+    # the untimed batch of the C ABI (deca_launch_timed without a result) computes what single
+    # launches do
+    y1, y2 = torch.empty_like(x), torch.full_like(x, float("nan"))
+    kern(x, y1)
+    kern.batch(kern.pack([(x, y2)]), 3)
+    torch.cuda.synchronize()
+    assert torch.equal(y1, y2)

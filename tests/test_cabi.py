@@ -29,7 +29,7 @@ def lib():
 def test_header_declares_entry_points():
     syms = declared_symbols()
     for name in ("deca_init", "deca_module_load", "deca_get_function", "deca_launch",
-                 "deca_launch_timed", "deca_module_unload", "deca_error_string",
+                 "deca_launch_timed", "deca_launch_between", "deca_module_unload", "deca_error_string",
                  "deca_device_info", "deca_set_max_dynamic_lds"):
         assert name in syms
 

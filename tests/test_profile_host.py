@@ -4,6 +4,8 @@ import csv
 import json
 import os
 
+import pytest
+
 from deca_amd.arch import profile
 
 
@@ -18,12 +20,11 @@ def _write(path, header, rows):
 def _passes(tmp, workload, dur_ns, steps=4, rowwise=False):
     out = str(tmp / f"prof_{workload}")
     n = steps * (3 if rowwise else 2)
-    # the event-timed launches take dur_ns, everything else twice as long
+    first = steps  # warm-up launches before, the pass over one buffer set after
+    # the timed launches take dur_ns, everything else twice as long
     trace = []
     for i in range(n):
-        last = steps * (2 if rowwise else 1)
-        timed = n - last <= i < n - last + steps
-        d = dur_ns if timed else 2 * dur_ns
+        d = dur_ns if first <= i < first + steps else 2 * dur_ns
         trace.append(["deca_main", 1000 * i * 10, 1000 * i * 10 + d])
     trace.append(["void at::native::fill", 5, 50])
     _write(os.path.join(out, "trace", "out_kernel_trace.csv"),
@@ -47,7 +48,8 @@ def _passes(tmp, workload, dur_ns, steps=4, rowwise=False):
                [[d, "deca_main", c, v, 100, 100 + dur_ns] for d in range(2) for c, v in vals.items()])
     work = 268435456 if rowwise else 1099511627776
     rec = {"steps": steps, "config": {"workload": workload, "kernel_config": "Br=256,mfma=16"},
-           "roofline": {"kernel_us": dur_ns / 1e3, "all": {workload: {"work": work}}}}
+           "roofline": {"kernel_us": dur_ns / 1e3, "timed_launches": [first, steps],
+                        "all": {workload: {"work": work}}}}
     with open(os.path.join(out, "trace.log"), "w") as f:
         f.write("[bench] noise\n" + json.dumps(rec) + "\n")
     return out
@@ -91,7 +93,11 @@ def test_summary_and_traffic_table(tmp_path):
     path = profile.summarise("softmax_fp16_16384x4096", out, str(prof_dir), traffic)
     text = open(path).read()
     assert os.path.basename(path) == "rowwise_softmax_fp16_16384x4096.md"
-    assert "average 42000 ns (min 42000, max 42000)" in text  # the event-timed launches only
+    assert "average 42000 ns (min 42000, max 42000)" in text  # the timed launches only
+    trace = profile._rows(os.path.join(out, "trace", "out_kernel_trace.csv"))
+    assert profile.event_timed_durations(trace, 0, 4) == [84000] * 4
+    with pytest.raises(ValueError):
+        profile.event_timed_durations(trace, 10, 4)
     assert "python -m deca_amd.arch.profile run softmax_fp16_16384x4096" in text
     assert "Matrix pipe" not in text
     entry = json.load(open(traffic))["workloads"]["softmax_fp16_16384x4096"]
