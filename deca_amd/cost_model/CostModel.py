@@ -378,8 +378,12 @@ def fa_score(cfg, arch, shape, causal: bool = False) -> float:
     # no max of the tile ahead of its exponentials (plain ring loops): +3.6 % on the full
     # S = 4096 shapes at both head dims; under the causal mask nothing is gained and the
     # second pass the step keeps in reserve costs 4-7 %
+    # (16x16x32 tiles then also take the row sums on the matrix pipe: another +3.9 % at D = 64,
+    # +1.2 % at D = 128)
     if getattr(cfg, "trust", False):
         pipe *= 1.035 if not causal else 0.95
+        if getattr(cfg, "mfma", 32) == 16 and not causal:
+            pipe *= 1.035 if D < 128 else 1.01
     if not getattr(cfg, "swizzle", True):
         pipe *= 0.5  # linear LDS rows: every fragment read is a multi-way bank conflict
     sync = 1.0 / (1.0 + getattr(arch, "fa_cta_sync_penalty", 0.0) * cfg.num_warps / 4 / wgs)

@@ -92,6 +92,11 @@
 #ifndef DECA_TRUST
 #define DECA_TRUST 0
 #endif
+// In the 16x16x32 form the trusted loops take a tile's row sums on the matrix pipe (one more
+// product per k-step, with a ones operand: four accumulator registers per query tile), which
+// frees the vector ALU of one add per score; l is then the sum of the fp16 P that the second
+// product also sees, already reduced over the lanes of a query.
+#define DECA_MFMASUM (DECA_TRUST && DECA_MFMA16)
 #ifndef DECA_MIN_WAVES
 #define DECA_MIN_WAVES 1  // waves per SIMD the register allocation must leave room for
 #endif
@@ -609,7 +614,8 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
 #if DECA_TRUST
   // The softmax of a tile taken on trust (`with_max` false): exponentials against the
   // running max as it stands, no max of the tile at all.  A lane's p are then bounded by
-  // their own sum, which is looked at afterwards: while no lane of the wave has more than
+  // their own sum (16x16x32 form: by the query's sum over the whole tile, which the matrix
+  // pipe delivers), which is looked at afterwards: while no lane of the wave has more than
   // 2^15 in it, every p fits fp16 and the running max may stay (alpha = 1, nothing to
   // rescale); otherwise the call returns true with l and O untouched, and the caller
   // computes S^T again and comes back with `with_max` true, which is `softmax` above.
@@ -643,7 +649,9 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
         for (int e = 0; e < ACC_N; ++e) {
           const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s_acc[kt][mq][e], SL2, -msl));
           s_acc[kt][mq][e] = p;
+#if !DECA_MFMASUM
           sum += p;
+#endif
         }
 #if !DECA_MFMA16
 #pragma unroll
@@ -666,6 +674,21 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
         }
         pf[kk][mq] = h;
       }
+#if DECA_MFMASUM
+      {
+        // the row sum on the matrix pipe: ones^T P^T has the sum over all keys of the tile
+        // in every row of a query's column (already reduced over the lanes of the query)
+        half8 ones;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) ones[e] = (_Float16)1.0f;
+        acc_t t;
+#pragma unroll
+        for (int e = 0; e < ACC_N; ++e) t[e] = 0.0f;
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) t = DECA_MFMA(ones, pf[kk][mq], t, 0, 0, 0);
+        sum = t[0];
+      }
+#endif
 #endif
       tile_sum[mq] = sum;
       over |= !(sum <= 32768.0f);  // also true for inf and NaN
@@ -1264,7 +1287,11 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
   _Float16* o_lds = reinterpret_cast<_Float16*>(lds) + wave * WQ * EPI_LD;
 #pragma unroll
   for (int mq = 0; mq < MQ; ++mq) {
+#if DECA_MFMASUM
+    const float l = l_i[mq];  // the matrix pipe's sums are already over all lanes of the query
+#else
     const float l = sum_over_query(l_i[mq]);
+#endif
     const float inv = 1.0f / l;
     // (16x16x32: o_acc[dt][mq][e]: q = mq*16 + lane%16, d = dt*16 + (lane/16)*4 + e)
     _Float16* o_row = EPI_LDS ? o_lds + (mq * TQ + lq) * EPI_LD + lg * 4

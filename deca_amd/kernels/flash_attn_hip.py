@@ -66,7 +66,10 @@ class FAConfig:
     # lanes of a query and the update arithmetic).  A lane's p are bounded by their own sum,
     # which is checked before the second product: a tile that outgrew the running max (the
     # first one always takes its max) is computed again with it.  Same quotient O / l.
-    # Measured: +3.6 % at D = 64 and D = 128 (S = 4096, full); nothing with the causal mask.
+    # In the 16x16x32 form the row sums of these loops are taken on the matrix pipe (one more
+    # product per k-step with a ones operand) instead of by one add per score.
+    # Measured: +3.6 % at D = 64 and D = 128 (S = 4096, full), the matrix-pipe sums another
+    # +3.9 % / +1.2 %; nothing with the causal mask.
     trust: bool = False
 
     @property

@@ -64,7 +64,7 @@ def attention_f32(q, k, v, scale=None, causal=False) -> np.ndarray:
 
 def flash_blockwise(q, k, v, scale=None, causal=False, Br=128, Bc=64, lazy_tau=0.0,
                     max_every=1, trust_bound=None, wave_rows=32, key_groups=(8, 4),
-                    stats=None) -> np.ndarray:
+                    sum_p16=False, stats=None) -> np.ndarray:
     """The tiled online-softmax recurrence; returns fp32 values rounded to fp16.
 
     `lazy_tau` = 0 is the reference's update m' = max(m, rowmax S)
@@ -81,9 +81,12 @@ def flash_blockwise(q, k, v, scale=None, causal=False, Br=128, Bc=64, lazy_tau=0
     taken against the running max as it stands, without its own max.  The p of a lane are
     bounded by their sum, so a wave (`wave_rows` query rows) accepts the tile while no lane's
     sum exceeds the bound -- a lane holds the keys k of the tile with
-    (k % key_groups[0]) // key_groups[1] == its group: (8, 4) for 32x32x16 tiles, (16, 4) for
-    16x16x32 -- and otherwise does the tile again with its max (lazy rule).  `stats`, a dict,
-    receives the number of (wave, tile) pairs taken on trust and of those done again."""
+    (k % key_groups[0]) // key_groups[1] == its group: (8, 4) for 32x32x16 tiles; `None` is one
+    group, the sum over the whole tile -- and otherwise does the tile again with its max (lazy
+    rule).  The kernel's 16x16x32 form takes these sums on the matrix pipe: over the whole
+    tile (`key_groups=None`) and of the fp16 P that the second product sees (`sum_p16`),
+    which is then also what l accumulates.  `stats`, a dict, receives the number of
+    (wave, tile) pairs taken on trust and of those done again."""
     q = np.asarray(q, np.float32)
     k = np.asarray(k, np.float32)
     v = np.asarray(v, np.float32)
@@ -114,9 +117,14 @@ def flash_blockwise(q, k, v, scale=None, causal=False, Br=128, Bc=64, lazy_tau=0
                     if trust_bound is not None and tile > 0:
                         # per wave: trust the running max unless the tile needs the mask or a
                         # lane's sum of p = exp2((s - m) sl2) says that some p may not fit fp16
-                        group = (np.arange(s.shape[1]) % key_groups[0]) // key_groups[1]
+                        if key_groups is None:
+                            group = np.zeros(s.shape[1], np.int64)
+                        else:
+                            group = (np.arange(s.shape[1]) % key_groups[0]) // key_groups[1]
                         with np.errstate(over="ignore"):
                             p_old = np.exp2(s * sl2 - (m * sl2)[:, None], dtype=np.float32)
+                            if sum_p16:
+                                p_old = p_old.astype(np.float16).astype(np.float32)
                         for w0 in range(0, s.shape[0], wave_rows):
                             w = slice(w0, w0 + wave_rows)
                             if causal and k0 + s.shape[1] - 1 > q0 + w0:
@@ -131,8 +139,8 @@ def flash_blockwise(q, k, v, scale=None, causal=False, Br=128, Bc=64, lazy_tau=0
                                 stats["redone"] = stats.get("redone", 0) + 1
                     alpha = np.exp2((m - m_new) * sl2, dtype=np.float32)
                     p = np.exp2(s * sl2 - (m_new * sl2)[:, None], dtype=np.float32)
-                    l = l * alpha + p.sum(axis=-1, dtype=np.float32)
                     p16 = p.astype(np.float16).astype(np.float32)
+                    l = l * alpha + (p16 if sum_p16 else p).sum(axis=-1, dtype=np.float32)
                     o = o * alpha[:, None] + p16 @ v[b, h, k0:k0 + Bc]
                     m = m_new
                 out[b, h, q0:q0 + Br] = o / l[:, None]

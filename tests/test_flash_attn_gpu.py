@@ -141,7 +141,7 @@ def test_flash_attn_trusted_max_is_outgrown(mfma, causal):
     st = {}
     want = oa.flash_blockwise(_f32(q), _f32(kr), _f32(v), None, causal, Br=cfg.Br, Bc=cfg.Bc, lazy_tau=8.0,
                               trust_bound=2.0 ** 15, wave_rows=cfg.Br // cfg.num_warps,
-                              key_groups=(16, 4) if mfma == 16 else (8, 4), stats=st)
+                              key_groups=None if mfma == 16 else (8, 4), sum_p16=mfma == 16, stats=st)
     assert st["redone"] > 0
     ref = oa.attention_f32(_f32(q), _f32(kr), _f32(v), None, causal)
     got = _f32(_run(B, H, S, S, D, causal, cfg, q, kr, v))

@@ -74,7 +74,7 @@ def test_running_max_must_see_every_tile():
     assert (s.reshape(64, 16, 32).max(-1)[:, 1:] - seen[:, :-1]).max() > 16 + 8
 
 
-@pytest.mark.parametrize("groups", [(8, 4), (16, 4)])
+@pytest.mark.parametrize("groups", [(8, 4), None])
 def test_trusted_running_max_is_checked_after_the_fact(groups):
     """`FAConfig.trust`: a tile's exponentials against the running max as it stands, without
     the tile's own max.  What makes that safe is the check behind it -- a lane's p are bounded
@@ -89,7 +89,7 @@ def test_trusted_running_max_is_checked_after_the_fact(groups):
         ref = oa.attention_f32(q, kk, vv, None, causal)
         st = {}
         got = oa.flash_blockwise(q, kk, vv, None, causal, Br=64, Bc=32, lazy_tau=8.0, trust_bound=2.0 ** 15,
-                                 key_groups=groups, stats=st)
+                                 key_groups=groups, sum_p16=groups is None, stats=st)
         assert np.abs(got - ref).max() < 2e-3
         assert st["trusted"] > 0 and st.get("redone", 0) == 0
     # growing keys: the running max is outgrown again and again
@@ -100,9 +100,9 @@ def test_trusted_running_max_is_checked_after_the_fact(groups):
     st = {}
     with np.errstate(over="ignore", invalid="ignore"):
         checked = oa.flash_blockwise(q, k, v, None, False, Br=64, Bc=32, lazy_tau=8.0, trust_bound=2.0 ** 15,
-                                     key_groups=groups, stats=st)
+                                     key_groups=groups, sum_p16=groups is None, stats=st)
         blind = oa.flash_blockwise(q, k, v, None, False, Br=64, Bc=32, lazy_tau=8.0, trust_bound=np.inf,
-                                   key_groups=groups)
+                                   key_groups=groups, sum_p16=groups is None)
     assert np.abs(checked - ref).max() < 2e-3
     assert 0 < st["redone"] < st["trusted"]
     assert not np.isfinite(blind).all() or np.abs(blind - ref).max() > 2e-3
