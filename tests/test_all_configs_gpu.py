@@ -23,6 +23,7 @@ EVERY = os.environ.get("DECA_ALL_CONFIGS") == "1"
 GEMM_STRIDE = int(os.environ.get("DECA_ALL_CONFIGS_GEMM_STRIDE", "7"))  # 1: every GEMM config
 GEMM_MFMA = os.environ.get("DECA_ALL_CONFIGS_GEMM_MFMA")  # "16" / "32": only that MFMA tile form
 GEMM_AGPR = os.environ.get("DECA_ALL_CONFIGS_GEMM_AGPR")  # "1" / "0": only configs with / without agpr
+FA_TRUST = os.environ.get("DECA_ALL_CONFIGS_FA_TRUST")  # "1" / "0": only attention configs with / without trust
 
 
 def gemm_configs(M, N, K):
@@ -122,6 +123,8 @@ def test_every_flash_attn_config(B, H, S, D, causal):
     configs = Solver.solve_flash_attn(_arch(), B, H, S, S, D)
     if not EVERY:
         configs = solver_sample(configs)
+    elif FA_TRUST:
+        configs = [c for c in configs if c.trust == (FA_TRUST == "1")]
     specs = [make_flash_attn_fwd(B, H, S, S, D, cfg, None, causal) for cfg in configs]
     paths = _build_all(specs)
     q, k, v = make_qkv(B, H, S, S, D)
