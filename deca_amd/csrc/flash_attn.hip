@@ -92,11 +92,15 @@
 #ifndef DECA_TRUST
 #define DECA_TRUST 0
 #endif
-// In the 16x16x32 form the trusted loops take a tile's row sums on the matrix pipe (one more
+// In the 16x16x32 form the plain loops take a tile's row sums on the matrix pipe (one more
 // product per k-step, with a ones operand: four accumulator registers per query tile), which
 // frees the vector ALU of one add per score; l is then the sum of the fp16 P that the second
-// product also sees, already reduced over the lanes of a query.
-#define DECA_MFMASUM (DECA_TRUST && DECA_MFMA16)
+// product also sees, already reduced over the lanes of a query.  (Not the slot loop, whose
+// slots carry the adds, nor the plain steps that finish its causal form: l has one meaning
+// per kernel.)
+#ifndef DECA_MFMASUM
+#define DECA_MFMASUM (DECA_MFMA16 && DECA_PIPE == 0)
+#endif
 #ifndef DECA_MIN_WAVES
 #define DECA_MIN_WAVES 1  // waves per SIMD the register allocation must leave room for
 #endif
@@ -573,7 +577,9 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
         for (int e = 0; e < ACC_N; ++e) {
           const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s_acc[kt][mq][e], SL2, -msl));
           s_acc[kt][mq][e] = p;
+#if !DECA_MFMASUM
           sum += p;
+#endif
         }
 #if !DECA_MFMA16
 #pragma unroll
@@ -596,6 +602,19 @@ deca_main(const _Float16* __restrict__ Q, const _Float16* __restrict__ K,
         }
         pf[kk][mq] = h;
       }
+#if DECA_MFMASUM
+      {
+        half8 ones;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) ones[e] = (_Float16)1.0f;
+        acc_t t;
+#pragma unroll
+        for (int e = 0; e < ACC_N; ++e) t[e] = 0.0f;
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) t = DECA_MFMA(ones, pf[kk][mq], t, 0, 0, 0);
+        sum = t[0];
+      }
+#endif
 #endif
       l_i[mq] = l_i[mq] * alpha[mq] + sum;
     }

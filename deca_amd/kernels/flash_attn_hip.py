@@ -48,7 +48,10 @@ class FAConfig:
     # before the softmax of tile j (two S^T accumulators).  2: as 1, and every matrix
     # instruction of an iteration carries a fixed share of its vector work.
     pipe: int = 0
-    # MFMA tile: 32 -> v_mfma_f32_32x32x16, 16 -> v_mfma_f32_16x16x32 (plain and slot loop)
+    # MFMA tile: 32 -> v_mfma_f32_32x32x16, 16 -> v_mfma_f32_16x16x32 (plain and slot loop).
+    # The plain loops on 16x16x32 tiles take the row sums on the matrix pipe (one more product
+    # per k-step with a ones operand) instead of by one add per score: +3.9 % / +1.2 % for the
+    # trusted winners of D = 64 / 128, +1 % for the rolled causal loop at D = 128.
     mfma: int = 32
     # Plain loop over two LDS stages: False unrolls it by two (each copy of the step knows its
     # ring slot and the scheduler overlaps the end of one step with the start of the next),
@@ -66,10 +69,7 @@ class FAConfig:
     # lanes of a query and the update arithmetic).  A lane's p are bounded by their own sum,
     # which is checked before the second product: a tile that outgrew the running max (the
     # first one always takes its max) is computed again with it.  Same quotient O / l.
-    # In the 16x16x32 form the row sums of these loops are taken on the matrix pipe (one more
-    # product per k-step with a ones operand) instead of by one add per score.
-    # Measured: +3.6 % at D = 64 and D = 128 (S = 4096, full), the matrix-pipe sums another
-    # +3.9 % / +1.2 %; nothing with the causal mask.
+    # Measured: +3.6 % at D = 64 and D = 128 (S = 4096, full); nothing with the causal mask.
     trust: bool = False
 
     @property

@@ -83,7 +83,7 @@ def flash_blockwise(q, k, v, scale=None, causal=False, Br=128, Bc=64, lazy_tau=0
     sum exceeds the bound -- a lane holds the keys k of the tile with
     (k % key_groups[0]) // key_groups[1] == its group: (8, 4) for 32x32x16 tiles; `None` is one
     group, the sum over the whole tile -- and otherwise does the tile again with its max (lazy
-    rule).  The kernel's 16x16x32 form takes these sums on the matrix pipe: over the whole
+    rule).  The kernel's plain loops on 16x16x32 tiles take these sums on the matrix pipe: over the whole
     tile (`key_groups=None`) and of the fp16 P that the second product sees (`sum_p16`),
     which is then also what l accumulates.  `stats`, a dict, receives the number of
     (wave, tile) pairs taken on trust and of those done again."""
