@@ -97,7 +97,7 @@
 // frees the vector ALU of one add per score; l is then the sum of the fp16 P that the second
 // product also sees, already reduced over the lanes of a query.  (Not the slot loop, whose
 // slots carry the adds, nor the plain steps that finish its causal form: l has one meaning
-// per kernel.)
+// per kernel.)  -DDECA_MFMASUM=0 builds the vector-ALU sums instead, for comparisons.
 #ifndef DECA_MFMASUM
 #define DECA_MFMASUM (DECA_MFMA16 && DECA_PIPE == 0)
 #endif
